@@ -1,0 +1,176 @@
+"""ctypes binding of the C ABI declared in include/blocked_attention.h.
+
+Thin and explicit: torch tensors are used only as device memory (``data_ptr``)
+and for the current HIP stream.  There is no CPU fallback: if the shared
+library is missing or a call fails, an exception is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libblockedattn_hip.so")
+
+BA_F16, BA_BF16, BA_F32 = 0, 1, 2
+META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
+
+SYMBOLS = (
+    "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
+    "ba_varlen_gemm", "ba_blocked_softmax", "ba_gemm_softmax",
+)
+
+
+class PlanInfo(ctypes.Structure):
+    _fields_ = [
+        ("nseg", ctypes.c_int64), ("Dm1", ctypes.c_int64), ("Dm2", ctypes.c_int64), ("Dout", ctypes.c_int64),
+        ("total_rows", ctypes.c_int64), ("gemm_items", ctypes.c_int64), ("strip_items", ctypes.c_int64),
+        ("split_items", ctypes.c_int64), ("wide_items", ctypes.c_int64), ("pack_items", ctypes.c_int64),
+        ("slow_items", ctypes.c_int64),
+        ("max_M", ctypes.c_int32), ("max_N", ctypes.c_int32), ("max_K", ctypes.c_int32),
+        ("bad_segments", ctypes.c_int32), ("run_errors", ctypes.c_int32), ("reserved", ctypes.c_int32),
+    ]
+
+    def as_dict(self):
+        return {name: getattr(self, name) for name, _ in self._fields_ if name != "reserved"}
+
+
+class BlockedAttentionError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load():
+    """Load libblockedattn_hip.so (built by ``python -m blockedattention_amd.build``)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise BlockedAttentionError(
+            f"{LIB_PATH} is missing: build it with `python -m blockedattention_amd.build lib` "
+            "(there is no CPU or PyTorch fallback)")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+    lib.ba_status_string.restype = ctypes.c_char_p
+    lib.ba_status_string.argtypes = [i32]
+    lib.ba_abi_version.restype = i32
+    lib.ba_plan_bytes.restype = ctypes.c_size_t
+    lib.ba_plan_bytes.argtypes = [i64]
+    lib.ba_plan_gemm.restype = i32
+    lib.ba_plan_gemm.argtypes = [vp, ctypes.c_size_t, i64, i32, vp, vp, vp, vp, vp, vp, vp]
+    lib.ba_plan_softmax.restype = i32
+    lib.ba_plan_softmax.argtypes = [vp, ctypes.c_size_t, i64, vp, vp, vp, i32, vp]
+    lib.ba_plan_read.restype = i32
+    lib.ba_plan_read.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
+    lib.ba_varlen_gemm.restype = i32
+    lib.ba_varlen_gemm.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
+    lib.ba_blocked_softmax.restype = i32
+    lib.ba_blocked_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, i64, i64, f32, vp]
+    lib.ba_gemm_softmax.restype = i32
+    lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
+    _lib = lib
+    return lib
+
+
+def check(status, what):
+    if status != 0:
+        raise BlockedAttentionError(f"{what}: {load().ba_status_string(status).decode()} (status {status})")
+
+
+def dtype_code(dtype):
+    try:
+        return {torch.float16: BA_F16, torch.bfloat16: BA_BF16, torch.float32: BA_F32}[dtype]
+    except KeyError:
+        raise BlockedAttentionError(f"unsupported dtype {dtype}") from None
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _meta(t, n, name):
+    if t is None:
+        return None
+    if t.dtype != torch.int64 or not t.is_cuda or not t.is_contiguous() or t.numel() != n:
+        raise BlockedAttentionError(f"{name} must be a contiguous int64 device tensor with {n} entries")
+    return t
+
+
+class Plan:
+    """Device-resident schedule for one batch of segments (see ba_plan_gemm / ba_plan_softmax)."""
+
+    def __init__(self, nseg, device):
+        self.nseg = int(nseg)
+        self.bytes = load().ba_plan_bytes(self.nseg)
+        self.buf = torch.empty(self.bytes, dtype=torch.uint8, device=device)
+        self.info = None
+
+    @property
+    def ptr(self):
+        return ctypes.c_void_p(self.buf.data_ptr())
+
+    def read(self, raise_on_bad=True):
+        """Blocking: copy the plan summary to the host (and remember it as the launch hint)."""
+        info = PlanInfo()
+        st = load().ba_plan_read(self.ptr, ctypes.byref(info), _stream())
+        if st != 0 and (raise_on_bad or st != 5):
+            check(st, "ba_plan_read")
+        self.info = info
+        return info
+
+    def _hint(self):
+        return ctypes.byref(self.info) if self.info is not None else None
+
+
+def plan_gemm(nseg, device, MList=None, NList=None, KList=None, accum1=None, accum2=None, accumOut=None,
+              mode=None):
+    """Run the scheduler.  Tensors passed as None in an *output* role are not written."""
+    have_lists = MList is not None and NList is not None and KList is not None
+    have_accum = accum1 is not None and accum2 is not None and accumOut is not None
+    if mode is None:
+        mode = META_GIVEN if (have_lists and have_accum) else (META_FROM_LISTS if have_lists else META_FROM_ACCUM)
+    for t, n, name in ((MList, nseg, "MList"), (NList, nseg, "NList"), (KList, nseg, "KList"),
+                       (accum1, nseg + 1, "mat1Accum"), (accum2, nseg + 1, "mat2Accum"),
+                       (accumOut, nseg + 1, "outAccum")):
+        _meta(t, n, name)
+    plan = Plan(nseg, device)
+    st = load().ba_plan_gemm(plan.ptr, plan.bytes, nseg, mode, _ptr(MList), _ptr(NList), _ptr(KList),
+                             _ptr(accum1), _ptr(accum2), _ptr(accumOut), _stream())
+    check(st, "ba_plan_gemm")
+    return plan
+
+
+def plan_softmax(nseg, device, rowList, colList, accum=None, accum_given=False):
+    _meta(rowList, nseg, "rowList"); _meta(colList, nseg, "colList"); _meta(accum, nseg + 1, "srcAccum")
+    plan = Plan(nseg, device)
+    st = load().ba_plan_softmax(plan.ptr, plan.bytes, nseg, _ptr(rowList), _ptr(colList), _ptr(accum),
+                                int(bool(accum_given)), _stream())
+    check(st, "ba_plan_softmax")
+    return plan
+
+
+def varlen_gemm(plan, A, B, out, H, Dm1, Dm2, Dout, transpose1=False, transpose2=False):
+    st = load().ba_varlen_gemm(plan.ptr, plan._hint(), dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out), H, Dm1, Dm2,
+                               Dout, int(transpose1), int(transpose2), _stream())
+    check(st, "ba_varlen_gemm")
+    return out
+
+
+def blocked_softmax(plan, src, dst, H, Dsrc, scale=1.0):
+    st = load().ba_blocked_softmax(plan.ptr, plan._hint(), dtype_code(src.dtype), _ptr(src), _ptr(dst), H, Dsrc,
+                                   float(scale), _stream())
+    check(st, "ba_blocked_softmax")
+    return dst
+
+
+def gemm_softmax(plan, A, B, out, H, Dm1, Dm2, Dout, scale=1.0):
+    st = load().ba_gemm_softmax(plan.ptr, plan._hint(), dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out),
+                                dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
+    check(st, "ba_gemm_softmax")
+    return out

@@ -1,0 +1,41 @@
+// Host-side declarations shared by the translation units of libblockedattn_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "../../include/blocked_attention.h"
+#include "ba_plan.hpp"
+
+namespace ba {
+
+// Flags passed to the compute kernels.
+enum RunFlags : int {
+    kFlagTranspose1 = 1,   // A segments stored K x M
+    kFlagTranspose2 = 2,   // B segments stored K x N
+    kFlagMfmaOk = 4,       // layouts, base pointers and head strides allow 16-byte operand loads
+    kFlagOutF32 = 8        // fused path writes fp32 probabilities
+};
+
+struct RunArgs {
+    void *plan;
+    const void *A;
+    const void *B;
+    void *out;
+    int64_t H, Dm1, Dm2, Dout;
+    float scale;
+    int flags;
+};
+
+int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,
+                    int64_t *K, int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream);
+
+// mode 0 = GEMM only, 1 = fused GEMM + softmax.  dtype BA_F16 / BA_BF16.
+// info: optional host copy of the plan summary (from ba_plan_read), or nullptr.
+int launch_strips(int dtype, int fused, const RunArgs &args, const ba_plan_info *info, hipStream_t stream);
+int launch_gemm_f32(const RunArgs &args, const ba_plan_info *info, hipStream_t stream);
+int launch_softmax(int dtype, void *plan, const void *src, void *dst, int64_t H, int64_t Dsrc, float scale,
+                   const ba_plan_info *info, hipStream_t stream);
+
+// Number of compute units of the current device (cached per device).
+int device_cu_count();
+
+}  // namespace ba

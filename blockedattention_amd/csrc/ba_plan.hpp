@@ -1,0 +1,91 @@
+// Plan: the device-resident result of the segment scheduler.  One contiguous
+// buffer; every compute kernel takes only this pointer plus the data pointers.
+//
+//   PlanHeader                                   (256 bytes)
+//   int64 off1[cap+1] off2[cap+1] offO[cap+1]    exclusive prefix sums (elements)
+//   int32 M[cap] N[cap] K[cap]                   segment shapes
+//   int32 prefix arrays, each [cap+1]            scanned work-item counts
+//
+// cap = nseg rounded up so that every array starts 16-byte aligned.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace ba {
+
+constexpr uint32_t kPlanMagic = 0xB10CA77Eu;
+constexpr int kStripRows = 16;    // rows of one work item (one MFMA tile high)
+constexpr int kWaveCols = 256;    // columns one wavefront keeps in registers (16 MFMA tiles)
+constexpr int kWavesPerGroup = 16;
+constexpr int kSplitCols = kWaveCols * kWavesPerGroup;  // 4096: columns one workgroup keeps in registers
+constexpr int kPackDim = 16;      // a pack of tiny segments fits one 16x16 MFMA tile
+
+// Kinds of scanned work-item counts.  Every kind except kPfxRows and kPfxSlow
+// counts aligned segments only (see below).
+enum PrefixKind {
+    kPfxGemm = 0,   // GEMM only: ceil(M/16) * ceil(N/256) per segment
+    kPfxStrip = 1,  // fused, N <= 256 and not packed: ceil(M/16)
+    kPfxSplit = 2,  // fused, 256 < N <= 4096: ceil(M/16)
+    kPfxWide = 3,   // fused, N > 4096: ceil(M/16)
+    kPfxRows = 4,   // softmax: M rows
+    kPfxPack = 5,   // 1 for the first segment of a pack of tiny segments, else 0
+    kPfxSlow = 6,   // ceil(M/16) for segments the 16-byte operand loads cannot serve
+    kNumPrefix = 7
+};
+
+// A segment is "aligned" when K % 8 == 0 and its A and B offsets are multiples
+// of 8 elements: every operand row then starts on a 16-byte boundary (given
+// 16-byte aligned base pointers and per-head strides that are multiples of 8).
+// Only aligned segments are counted in kPfxGemm/Strip/Split/Wide/Pack; the
+// others are counted in kPfxSlow and take the element-wise path.
+
+struct PlanHeader {
+    uint32_t magic;
+    int32_t nseg;
+    int32_t cap;
+    int32_t kind;            // 0 = GEMM plan, 1 = softmax plan
+    int64_t Dm1, Dm2, Dout;
+    int64_t total_rows;
+    int64_t totals[8];       // last entry of each prefix array
+    int32_t max_M, max_N, max_K;
+    int32_t bad_segments;
+    int32_t run_errors;      // bumped by kernels that refuse to run
+    int32_t pad_[31];
+};
+static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
+
+__host__ __device__ inline int64_t plan_cap(int64_t nseg) { return (nseg + 4) & ~int64_t(3); }
+
+struct PlanView {
+    PlanHeader *hdr;
+    int64_t *off1, *off2, *offO;
+    int32_t *M, *N, *K;
+    int32_t *pfx[kNumPrefix];
+    // Segments that belong to a pack store the pack's segment count in packLen
+    // (leader) or 0 (follower / not packed).
+    int32_t *packLen;
+};
+
+__host__ __device__ inline size_t plan_bytes_for(int64_t nseg) {
+    const size_t cap = (size_t)plan_cap(nseg);
+    return sizeof(PlanHeader) + 3 * (cap + 4) * sizeof(int64_t) + 4 * cap * sizeof(int32_t) +
+           kNumPrefix * (cap + 4) * sizeof(int32_t);
+}
+
+__host__ __device__ inline PlanView plan_view(void *buf, int64_t nseg) {
+    PlanView v;
+    const size_t cap = (size_t)plan_cap(nseg);
+    char *p = (char *)buf;
+    v.hdr = (PlanHeader *)p; p += sizeof(PlanHeader);
+    v.off1 = (int64_t *)p; p += (cap + 4) * sizeof(int64_t);
+    v.off2 = (int64_t *)p; p += (cap + 4) * sizeof(int64_t);
+    v.offO = (int64_t *)p; p += (cap + 4) * sizeof(int64_t);
+    v.M = (int32_t *)p; p += cap * sizeof(int32_t);
+    v.N = (int32_t *)p; p += cap * sizeof(int32_t);
+    v.K = (int32_t *)p; p += cap * sizeof(int32_t);
+    v.packLen = (int32_t *)p; p += cap * sizeof(int32_t);
+    for (int i = 0; i < kNumPrefix; ++i) { v.pfx[i] = (int32_t *)p; p += (cap + 4) * sizeof(int32_t); }
+    return v;
+}
+
+}  // namespace ba

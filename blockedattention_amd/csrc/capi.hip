@@ -1,0 +1,138 @@
+// extern "C" entry points of libblockedattn_hip.so: argument checks, flag
+// derivation and kernel launches.  No allocation, no host synchronisation
+// except ba_plan_read.
+#include <string.h>
+
+#include "ba_host.hpp"
+
+namespace ba {
+
+int device_cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// The MFMA paths load operand rows 16 bytes at a time: that needs untransposed
+// layouts, 16-byte aligned base pointers and, with more than one head, per-head
+// strides that keep every head's rows aligned.  (Per-segment alignment is
+// settled by the scheduler.)
+static int mfma_flag(const RunArgs &r) {
+    if (r.flags & (kFlagTranspose1 | kFlagTranspose2)) return 0;
+    if ((((uintptr_t)r.A | (uintptr_t)r.B) & 15) != 0) return 0;
+    if (r.H > 1 && ((r.Dm1 | r.Dm2) & 7) != 0) return 0;
+    return kFlagMfmaOk;
+}
+
+static bool bad_sizes(int64_t H, int64_t d1, int64_t d2, int64_t d3) { return H < 0 || d1 < 0 || d2 < 0 || d3 < 0; }
+
+}  // namespace ba
+
+using namespace ba;
+
+extern "C" {
+
+__attribute__((visibility("default"))) const char *ba_status_string(int status) {
+    switch (status) {
+        case BA_OK: return "ok";
+        case BA_ERR_INVALID_ARG: return "invalid argument";
+        case BA_ERR_WORKSPACE: return "plan buffer too small or misaligned";
+        case BA_ERR_UNSUPPORTED: return "unsupported dtype or flag combination";
+        case BA_ERR_LAUNCH: return "HIP launch or copy failed";
+        case BA_ERR_BAD_METADATA: return "segment metadata rejected on the device";
+        default: return "unknown status";
+    }
+}
+
+__attribute__((visibility("default"))) int ba_abi_version(void) { return BA_ABI_VERSION; }
+
+__attribute__((visibility("default"))) size_t ba_plan_bytes(int64_t nseg) {
+    if (nseg < 0) return 0;
+    return (plan_bytes_for(nseg) + 255) & ~size_t(255);
+}
+
+__attribute__((visibility("default"))) int ba_plan_gemm(void *plan, size_t plan_bytes, int64_t nseg, int mode,
+                                                        int64_t *MList, int64_t *NList, int64_t *KList,
+                                                        int64_t *accum1, int64_t *accum2, int64_t *accumOut,
+                                                        ba_stream_t stream) {
+    return launch_schedule(plan, plan_bytes, nseg, mode, 0, MList, NList, KList, accum1, accum2, accumOut,
+                           (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_plan_softmax(void *plan, size_t plan_bytes, int64_t nseg,
+                                                           const int64_t *rowList, const int64_t *colList,
+                                                           int64_t *accum, int accum_given, ba_stream_t stream) {
+    return launch_schedule(plan, plan_bytes, nseg, accum_given ? BA_META_GIVEN : BA_META_FROM_LISTS, 1,
+                           const_cast<int64_t *>(rowList), const_cast<int64_t *>(colList), nullptr, nullptr,
+                           nullptr, accum, (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_plan_info *info, ba_stream_t stream) {
+    if (!plan || !info) return BA_ERR_INVALID_ARG;
+    PlanHeader h;
+    if (hipMemcpyAsync(&h, plan, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+        return BA_ERR_LAUNCH;
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return BA_ERR_LAUNCH;
+    if (h.magic != kPlanMagic) return BA_ERR_INVALID_ARG;
+    memset(info, 0, sizeof(*info));
+    info->nseg = h.nseg;
+    info->Dm1 = h.Dm1; info->Dm2 = h.Dm2; info->Dout = h.Dout;
+    info->total_rows = h.total_rows;
+    info->gemm_items = h.totals[kPfxGemm];
+    info->strip_items = h.totals[kPfxStrip];
+    info->split_items = h.totals[kPfxSplit];
+    info->wide_items = h.totals[kPfxWide];
+    info->pack_items = h.totals[kPfxPack];
+    info->slow_items = h.totals[kPfxSlow];
+    info->max_M = h.max_M; info->max_N = h.max_N; info->max_K = h.max_K;
+    info->bad_segments = h.bad_segments;
+    info->run_errors = h.run_errors;
+    return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
+}
+
+__attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_plan_info *info, int dtype,
+                                                          const void *A, const void *B, void *out, int64_t H,
+                                                          int64_t Dm1, int64_t Dm2, int64_t Dout, int transpose1,
+                                                          int transpose2, ba_stream_t stream) {
+    if (!plan || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dout == 0) return BA_OK;
+    if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0};
+    if (transpose1) args.flags |= kFlagTranspose1;
+    if (transpose2) args.flags |= kFlagTranspose2;
+    args.flags |= mfma_flag(args);
+    if (dtype == BA_F32) return launch_gemm_f32(args, info, (hipStream_t)stream);
+    return launch_strips(dtype, 0, args, info, (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_blocked_softmax(void *plan, const ba_plan_info *info, int dtype,
+                                                              const void *src, void *dst, int64_t H, int64_t Dsrc,
+                                                              float scale, ba_stream_t stream) {
+    if (!plan || H < 0 || Dsrc < 0) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dsrc == 0) return BA_OK;
+    if (!src || !dst) return BA_ERR_INVALID_ARG;
+    return launch_softmax(dtype, plan, src, dst, H, Dsrc, scale, info, (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_plan_info *info, int dtype,
+                                                           const void *A, const void *B, void *out, int out_dtype,
+                                                           int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
+                                                           float scale, ba_stream_t stream) {
+    if (!plan || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
+    if (out_dtype != dtype && out_dtype != BA_F32) return BA_ERR_UNSUPPORTED;
+    if (H == 0 || Dout == 0) return BA_OK;
+    if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0};
+    args.flags |= mfma_flag(args);
+    if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
+    return launch_strips(dtype, 1, args, info, (hipStream_t)stream);
+}
+
+}  // extern "C"

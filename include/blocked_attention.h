@@ -1,0 +1,155 @@
+/*
+ * blocked_attention.h -- C ABI of the MI355X (gfx950) varlen GEMM + blocked
+ * softmax library (libblockedattn_hip.so).
+ *
+ * Everything is plain pointers and sizes: no torch types, no C++ types, no
+ * exceptions.  All data and metadata pointers are DEVICE pointers unless a
+ * parameter says "host".  All entry points are stream-ordered on `stream` (a
+ * hipStream_t passed as void*; NULL is the null stream), return a ba_status
+ * and, except ba_plan_read, never synchronise with the host and never
+ * allocate: the only scratch is the caller-provided plan buffer.
+ *
+ * The reference (Sophie10001b/blockedAttention) has no C ABI; its boundary is
+ * a pybind11 torch extension.  Each entry point below names the reference
+ * interface it stands in for (paths relative to the reference checkout).
+ *
+ * Layout contract (csrc/cuda/spBlkGEMM.cu:133-150, 985-1008;
+ * csrc/cuda/spBlkSoftmax.cu:95-107, 375-398): operands are [H, D] row-major,
+ * segment g occupies [accum[g], accum[g+1]) of the last dimension, row-major
+ * inside the segment; head h of a buffer starts at h * D elements.
+ */
+#ifndef BLOCKED_ATTENTION_H
+#define BLOCKED_ATTENTION_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BA_ABI_VERSION 1
+
+typedef void *ba_stream_t; /* hipStream_t */
+
+typedef enum ba_status {
+    BA_OK = 0,
+    BA_ERR_INVALID_ARG = 1,  /* null pointer, negative size, unknown enum */
+    BA_ERR_WORKSPACE = 2,    /* plan buffer too small or misaligned */
+    BA_ERR_UNSUPPORTED = 3,  /* dtype / flag combination not built */
+    BA_ERR_LAUNCH = 4,       /* HIP reported an error at launch or copy */
+    BA_ERR_BAD_METADATA = 5  /* ba_plan_read: the device-side checks rejected segments */
+} ba_status;
+
+typedef enum ba_dtype { BA_F16 = 0, BA_BF16 = 1, BA_F32 = 2 } ba_dtype;
+
+/* Which half of the metadata the caller supplies
+ * (the three cases of csrc/sparseBlockedAttention.cpp:22-44). */
+typedef enum ba_meta_mode {
+    BA_META_FROM_LISTS = 0, /* lists are inputs, prefix sums are written   (cpp:22-29) */
+    BA_META_FROM_ACCUM = 1, /* prefix sums are inputs, lists are written   (cpp:30-40) */
+    BA_META_GIVEN = 2       /* both are inputs                             (cpp:41-44) */
+} ba_meta_mode;
+
+/* Host-visible summary of a plan (filled by ba_plan_read). */
+typedef struct ba_plan_info {
+    int64_t nseg;
+    int64_t Dm1, Dm2, Dout; /* last prefix-sum entries = elements per head */
+    int64_t total_rows;     /* sum of M */
+    int64_t gemm_items;     /* 16 x <=256 output pieces of the GEMM-only kernel */
+    int64_t strip_items;    /* 16-row strips with N <= 256 (one wavefront each) */
+    int64_t split_items;    /* 16-row strips with 256 < N <= 4096 (one workgroup each) */
+    int64_t wide_items;     /* 16-row strips with N > 4096 (two-sweep path) */
+    int64_t pack_items;     /* packs of tiny segments sharing one wavefront */
+    int64_t slow_items;     /* 16-row strips of segments that need the element-wise path */
+    int32_t max_M, max_N, max_K;
+    int32_t bad_segments;   /* segments rejected by the device-side checks */
+    int32_t run_errors;     /* kernels that refused to run against this plan */
+    int32_t reserved;
+} ba_plan_info;
+
+const char *ba_status_string(int status);
+int ba_abi_version(void);
+
+/* Bytes of device memory a plan for nseg segments needs (256-byte aligned
+ * buffer).  Depends on nseg only, so it can be sized without knowing any
+ * segment shape. */
+size_t ba_plan_bytes(int64_t nseg);
+
+/*
+ * Device-side segment scheduler for the GEMM (and the fused pair).
+ * Stands in for the metadata derivation of sparseBlockedGEMM::forward
+ * (csrc/sparseBlockedAttention.cpp:17-44) and for the host-side tile list of
+ * __getTiling (csrc/cuda/spBlkGEMM.cu:943-983): one kernel, no host round
+ * trip.  Depending on `mode` it reads or writes MList/NList/KList (int64[nseg])
+ * and accum1/accum2/accumOut (int64[nseg+1]); the plan receives offsets, sizes
+ * and the scanned work-item counts every compute kernel searches.
+ * In BA_META_FROM_ACCUM the lists are derived in exact integer arithmetic.
+ * Output pointers may be NULL when the caller does not need that half.
+ */
+int ba_plan_gemm(void *plan, size_t plan_bytes, int64_t nseg, int mode,
+                 int64_t *MList, int64_t *NList, int64_t *KList,
+                 int64_t *accum1, int64_t *accum2, int64_t *accumOut,
+                 ba_stream_t stream);
+
+/*
+ * Scheduler for the standalone softmax.  Stands in for
+ * sparseBlockedSoftmax::forward's prefix sum (csrc/sparseBlockedAttention.cpp:85-91)
+ * and the per-row list of __getTiling (csrc/cuda/spBlkSoftmax.cu:358-373).
+ * accum_given != 0: accum (int64[nseg+1]) is an input; else, if non-NULL, it is written.
+ */
+int ba_plan_softmax(void *plan, size_t plan_bytes, int64_t nseg,
+                    const int64_t *rowList, const int64_t *colList,
+                    int64_t *accum, int accum_given, ba_stream_t stream);
+
+/* Copies the plan summary to the host and waits for it (the one blocking
+ * call).  Returns BA_ERR_BAD_METADATA if the scheduler rejected any segment
+ * or a kernel refused to run against the plan.
+ *
+ * The compute entry points below take the summary back as `info` (a HOST
+ * pointer, may be NULL).  With it they launch exactly the kernels the plan has
+ * work for, with grids that cover the work; without it they launch every
+ * kernel with a resident-size grid and let the kernels read the counts from
+ * the plan, which costs a few extra (empty) launches but no synchronisation.
+ * The results are identical either way. */
+int ba_plan_read(const void *plan, ba_plan_info *host_info, ba_stream_t stream);
+
+/*
+ * out[h, accumOut[g] + r*N_g + c] = sum_t A(h,g,r,t) * B(h,g,c,t), one rounding
+ * to the operand dtype at the store.  Stands in for sparseBlockedGEMMLaunch
+ * (csrc/sparseBlockedAttention.h:18, csrc/cuda/spBlkGEMM.cu:985-1033).
+ * Dm1/Dm2/Dout are the per-head strides of A/B/out in elements and must equal
+ * the plan's totals, otherwise the kernel writes nothing and records a run
+ * error in the plan.  transpose1/transpose2 select the K x M / K x N segment
+ * layouts (spBlkGEMM.cu:292-329, 363-400).  dtype: BA_F16, BA_BF16 (MFMA,
+ * fp32 accumulate) or BA_F32.
+ */
+int ba_varlen_gemm(void *plan, const ba_plan_info *info, int dtype, const void *A, const void *B, void *out,
+                   int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
+                   int transpose1, int transpose2, ba_stream_t stream);
+
+/*
+ * dst row = softmax(scale * src row) for every row of every segment, computed
+ * in fp32, one rounding at the store.  Stands in for sparseBlockedSoftmaxLaunch
+ * (csrc/sparseBlockedAttention.h:20, csrc/cuda/spBlkSoftmax.cu:375-416);
+ * scale = 1.0f reproduces it.  No column limit.  src == dst is allowed.
+ */
+int ba_blocked_softmax(void *plan, const ba_plan_info *info, int dtype, const void *src, void *dst,
+                       int64_t H, int64_t Dsrc, float scale, ba_stream_t stream);
+
+/*
+ * Fused pair: out = softmax(scale * A_g B_g^T) per segment with the scores kept
+ * in fp32 registers between the two steps.  Equivalent to ba_varlen_gemm
+ * followed by ba_blocked_softmax on (M, N, accumOut) without the intermediate
+ * 16-bit rounding; it has no single counterpart in the reference (which offers
+ * only the two separate launchers above) and takes a plan from ba_plan_gemm.
+ * out_dtype: the operand dtype, or BA_F32 for fp32 probabilities.
+ */
+int ba_gemm_softmax(void *plan, const ba_plan_info *info, int dtype, const void *A, const void *B, void *out,
+                    int out_dtype, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout, float scale,
+                    ba_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BLOCKED_ATTENTION_H */
