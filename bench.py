@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the varlen QK^T + blocked softmax pair on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu] [--no-others]
+
+One step = one pass of the hot path over one batch of synthetic segments, as a
+caller of the C ABI issues it: the device-side scheduler (ba_plan_gemm) followed
+by the fused GEMM + softmax (ba_gemm_softmax), stream-ordered, no host
+synchronisation, operands and result resident in HBM.  The launch hint (the
+plan summary) is read once before the timed region, as a caller that reuses one
+graph batch across layers does.
+
+Prints ONE JSON line.  `value` is microseconds per call of that step
+(lower is better) on the configuration the metric is quoted on (config 2:
+256 segments x 8 heads, n ~ U[32,128], K = 64, fp16).  `roofline` is for the
+dominant kernel (the fused kernel) against the 8 TB/s HBM peak, with the
+algorithmic bytes "A and B read once, probabilities written once".
+`cpu_baseline` is the per-segment torch matmul + softmax path on the host cores.
+`others` carries the same GPU figures for the remaining configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=30)
+    p.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-others", action="store_true", help="skip the other configurations")
+    p.add_argument("--cpu-seconds", type=float, default=12.0)
+    return p.parse_args()
+
+
+class Case:
+    """One configuration resident on the GPU, with its plan."""
+
+    def __init__(self, cfg, dev):
+        import torch
+        from blockedattention_amd import capi, workloads
+        self.torch, self.capi = torch, capi
+        self.w = w = workloads.make(cfg)
+        self.cfg = cfg
+        A, B = w.operands()
+        self.A_host, self.B_host = A, B
+        self.A, self.B = A.to(dev), B.to(dev)
+        i64 = lambda a: torch.from_numpy(a).to(dev)
+        self.M, self.N, self.K = i64(w.M), i64(w.N), i64(w.K)
+        self.acc = [torch.empty(w.nseg + 1, dtype=torch.int64, device=dev) for _ in range(3)]
+        self.out = torch.empty((w.heads, w.Dout), dtype=w.dtype, device=dev)
+        self.scores = None
+        self.plan = capi.plan_gemm(w.nseg, dev, self.M, self.N, self.K, *self.acc, mode=capi.META_FROM_LISTS)
+        self.plan.read()
+        self.dev = dev
+
+    def schedule(self):
+        c, w, p = self.capi, self.w, self.plan
+        st = c.load().ba_plan_gemm(p.ptr, p.bytes, w.nseg, c.META_FROM_LISTS, c._ptr(self.M), c._ptr(self.N),
+                                   c._ptr(self.K), c._ptr(self.acc[0]), c._ptr(self.acc[1]), c._ptr(self.acc[2]),
+                                   c._stream())
+        c.check(st, "ba_plan_gemm")
+
+    def fused(self):
+        w = self.w
+        self.capi.gemm_softmax(self.plan, self.A, self.B, self.out, w.heads, w.Dm1, w.Dm2, w.Dout, w.scale)
+
+    def step(self):
+        self.schedule()
+        self.fused()
+
+    def unfused(self):
+        w = self.w
+        if self.scores is None:
+            self.scores = self.torch.empty_like(self.out)
+        self.capi.varlen_gemm(self.plan, self.A, self.B, self.scores, w.heads, w.Dm1, w.Dm2, w.Dout)
+        self.capi.blocked_softmax(self.plan, self.scores, self.out, w.heads, w.Dout, w.scale)
+
+    def event_us(self, fn, steps, warmup):
+        """Average device time of fn over `steps` back-to-back calls, HIP events on the launch stream."""
+        torch = self.torch
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    def wall_us(self, fn, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e6 / steps
+
+    def check(self):
+        """Parity gate before any number is reported: sampled segments against fp32 torch on the host."""
+        import numpy as np
+        torch, w = self.torch, self.w
+        self.step()
+        torch.cuda.synchronize()
+        a1 = self.acc[0].cpu().numpy(); a2 = self.acc[1].cpu().numpy(); ao = self.acc[2].cpu().numpy()
+        rng = np.random.default_rng(1)
+        worst = 0.0
+        for g in rng.choice(w.nseg, size=min(8, w.nseg), replace=False):
+            h = int(rng.integers(0, w.heads))
+            m, n, k = int(w.M[g]), int(w.N[g]), int(w.K[g])
+            a = self.A_host[h, a1[g]:a1[g + 1]].float().reshape(m, k)
+            b = self.B_host[h, a2[g]:a2[g + 1]].float().reshape(n, k)
+            ref = torch.softmax(a @ b.t() * w.scale, -1)
+            got = self.out[h, ao[g]:ao[g + 1]].float().cpu().reshape(m, n)
+            tol = 1e-3 + (ref * 2.0 ** -8 if w.dtype == torch.bfloat16 else 0)
+            err = (got - ref).abs()
+            if not bool((err <= tol).all()):
+                raise SystemExit(f"parity gate failed on config {self.cfg}, segment {g}, head {h}: {float(err.max())}")
+            worst = max(worst, float(err.max()))
+        return worst
+
+    def gpu_figures(self, steps, warmup, with_unfused=True):
+        w = self.w
+        k_us = self.event_us(self.fused, steps, warmup)
+        fig = {
+            "workload": w.name, "dtype": str(w.dtype).replace("torch.", ""),
+            "kernel_us": round(k_us, 3),
+            "call_us": round(self.wall_us(self.step, steps, warmup), 3),
+            "scheduler_us": round(self.event_us(self.schedule, steps, warmup), 3),
+            "pair_bytes": w.pair_bytes(), "flops": w.flops,
+            "GBps": round(w.pair_bytes() / k_us * 1e-3, 1), "TFLOPs": round(w.flops / k_us * 1e-6, 2),
+            "hbm_frac": round(w.pair_bytes() / k_us * 1e-3 / HBM_PEAK_GBS, 4),
+            "mfma_frac": round(w.flops / k_us * 1e-6 / MFMA_PEAK_TFLOPS, 4),
+        }
+        if with_unfused:
+            fig["unfused_pair_us"] = round(self.event_us(self.unfused, steps, warmup), 3)
+        return fig
+
+
+def cpu_baseline(case, seconds):
+    """Per-segment fp32 torch matmul + softmax on the host cores, bounded to about `seconds`."""
+    import torch
+    import oracle
+    w = case.w
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    heads = w.heads
+    A, B = case.A_host.float(), case.B_host.float()
+    t0 = time.perf_counter()
+    oracle.per_segment_torch(A[:1], B[:1], w.M, w.N, w.K, w.scale)       # warm-up on one head
+    one_head = time.perf_counter() - t0
+    use_heads = heads if one_head * heads < seconds / 2 else max(1, int(seconds / 2 / max(one_head, 1e-9)))
+    use_heads = min(use_heads, heads)
+    times = []
+    t_end = time.perf_counter() + seconds
+    while len(times) < 50 and (not times or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        oracle.per_segment_torch(A[:use_heads], B[:use_heads], w.M, w.N, w.K, w.scale)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2] * heads / use_heads
+    return {"value": round(med * 1e6, 1), "unit": "us/call", "cores": cores, "kind": "port",
+            "sample": f"{len(times)} run(s) of per-segment torch.matmul+softmax (fp32) over {use_heads} of {heads} "
+                      f"head(s) of {w.name}, median scaled to all heads"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path has no cross-GPU step (heads and segments are independent), "
+              "so --gpus must be 1", file=sys.stderr)
+        return 2
+    import torch
+    from blockedattention_amd import capi
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP library is the only compute path)", file=sys.stderr)
+        return 2
+    capi.load()
+    dev = torch.device("cuda:0")
+    case = Case(args.config, dev)
+    worst = case.check()
+    fig = case.gpu_figures(args.steps, args.warmup)
+    # the timed region of the contract: W warm-up steps, then exactly K steps between synchronisations
+    call_us = case.wall_us(case.step, args.steps, args.warmup)
+    w = case.w
+    line = {
+        "metric": "varlen QK^T+softmax us/call (scheduler + fused kernel, stream-ordered)",
+        "value": round(call_us, 3), "unit": "us/call", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(call_us * 1e-3, 6), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if w.dtype == torch.float16 else "bf16", "data": "synthetic",
+        "config": {"workload": w.name, "segments": w.nseg, "heads": w.heads, "seed": 0,
+                   "flops": w.flops, "pair_bytes": w.pair_bytes()},
+        "roofline": {"bound": "hbm", "achieved": fig["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": fig["hbm_frac"], "traffic": None, "kernel": "wave_items_kernel (fused)",
+                     "kernel_us": fig["kernel_us"], "mfma_frac": fig["mfma_frac"], "TFLOPs": fig["TFLOPs"]},
+        "parity_max_abs_err": worst,
+        "detail": fig,
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic_file):
+        try:
+            line["roofline"]["traffic"] = json.load(open(traffic_file)).get(w.name)
+        except (OSError, ValueError):
+            pass
+    try:
+        import blockedAttention
+        ML, NL, KL = case.M, case.N, case.K
+        op = lambda: blockedAttention.blockGEMMSoftmax(case.A, case.B, MList=ML, NList=NL, KList=KL, scale=w.scale)
+        line["detail"]["torch_op_us"] = round(case.wall_us(op, max(10, args.steps // 4), 5), 3)
+    except ImportError as e:
+        line["detail"]["torch_op_us"] = f"extension not built: {e}"
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(case, args.cpu_seconds)
+    if not args.no_others:
+        others = {}
+        del case
+        torch.cuda.empty_cache()
+        for cfg in (1, 2, 3, 4, 5):
+            if cfg == args.config:
+                continue
+            c = Case(cfg, dev)
+            err = c.check()
+            steps = args.steps if cfg != 5 else max(5, min(args.steps, 20))
+            f = c.gpu_figures(steps, min(args.warmup, steps), with_unfused=cfg != 5)
+            f["parity_max_abs_err"] = err
+            others[f"cfg{cfg}"] = f
+            del c
+            torch.cuda.empty_cache()
+        line["others"] = others
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

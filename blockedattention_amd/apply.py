@@ -1,0 +1,70 @@
+"""Python surface of the operators: the reference's ``blockGEMM`` and
+``blockSoftmax`` (blockedAttention/apply.py:6-41) with identical names,
+argument order and defaults, plus the fused pair.
+
+All three forward to the compiled extension ``blockAttention`` (built in-tree
+by ``python -m blockedattention_amd.build``); there is no Python or CPU
+fallback.  The reference wrapper passes ``srcAccum`` to the extension in the
+wrong position (apply.py:41 against csrc/sparseBlockedAttention.cpp:127-128);
+here the call follows the extension's order, so ``blockSoftmax(x, rows, cols)``
+works as documented.
+"""
+from typing import Optional
+
+import torch
+
+from . import blockAttention
+
+
+def blockGEMM(
+    mat1: torch.Tensor, mat2: torch.Tensor,
+    mat1Accum: Optional[torch.Tensor] = None, mat2Accum: Optional[torch.Tensor] = None,
+    outAccum: Optional[torch.Tensor] = None,
+    MList: Optional[torch.Tensor] = None, NList: Optional[torch.Tensor] = None, KList: Optional[torch.Tensor] = None,
+    transpose1: Optional[bool] = False, transpose2: Optional[bool] = False,
+) -> torch.Tensor:
+    """Varlen GEMM ``out_g = A_g @ B_g^T`` over segments stored back to back.
+
+    ``mat1`` is ``[H, sum(M_g*K_g)]``, ``mat2`` is ``[H, sum(N_g*K_g)]`` and the
+    result ``[H, sum(M_g*N_g)]``; segment ``g`` is row-major ``M_g x K_g``
+    (``K_g x M_g`` with ``transpose1``), ``N_g x K_g`` (``K_g x N_g`` with
+    ``transpose2``) and ``M_g x N_g``.  Give either the three exclusive prefix
+    sums (int64, one more entry than segments) or the three size lists (int64),
+    or both.
+    """
+    return blockAttention.sparseBlockedGEMM(mat1, mat2, mat1Accum, mat2Accum, outAccum, MList, NList, KList,
+                                            bool(transpose1), bool(transpose2))
+
+
+def blockSoftmax(
+    src: torch.Tensor,
+    rowList: torch.Tensor, colList: torch.Tensor, srcAccum: Optional[torch.Tensor] = None,
+    scale: float = 1.0,
+) -> torch.Tensor:
+    """Row softmax inside every ``rowList[g] x colList[g]`` block of ``src`` (``[H, sum(rows*cols)]``).
+
+    ``srcAccum`` (the exclusive prefix sum of ``rows*cols``) is optional.
+    ``scale`` multiplies the input first; the default 1.0 is the reference's
+    behaviour.
+    """
+    if scale == 1.0:
+        return blockAttention.sparseBlockedSoftmax(src, rowList, colList, srcAccum)
+    return blockAttention.sparseBlockedSoftmaxScaled(src, rowList, colList, srcAccum, float(scale))
+
+
+def blockGEMMSoftmax(
+    mat1: torch.Tensor, mat2: torch.Tensor,
+    mat1Accum: Optional[torch.Tensor] = None, mat2Accum: Optional[torch.Tensor] = None,
+    outAccum: Optional[torch.Tensor] = None,
+    MList: Optional[torch.Tensor] = None, NList: Optional[torch.Tensor] = None, KList: Optional[torch.Tensor] = None,
+    scale: float = 1.0, out_fp32: bool = False,
+) -> torch.Tensor:
+    """Fused ``softmax(scale * A_g @ B_g^T)`` per segment (forward only).
+
+    Same operands and metadata as ``blockGEMM`` (untransposed layouts); the
+    scores stay in fp32 registers between the product and the softmax, so the
+    result is what ``blockSoftmax(blockGEMM(...), MList, NList, scale=scale)``
+    computes without the intermediate 16-bit rounding.
+    """
+    return blockAttention.sparseBlockedGEMMSoftmax(mat1, mat2, mat1Accum, mat2Accum, outAccum, MList, NList, KList,
+                                                   float(scale), bool(out_fp32))

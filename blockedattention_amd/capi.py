@@ -17,7 +17,7 @@ META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
 
 SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
-    "ba_varlen_gemm", "ba_blocked_softmax", "ba_gemm_softmax",
+    "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax",
 )
 
 
@@ -68,6 +68,8 @@ def load():
     lib.ba_varlen_gemm.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
     lib.ba_blocked_softmax.restype = i32
     lib.ba_blocked_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, i64, i64, f32, vp]
+    lib.ba_blocked_softmax_backward.restype = i32
+    lib.ba_blocked_softmax_backward.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i64, i64, f32, vp]
     lib.ba_gemm_softmax.restype = i32
     lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
     _lib = lib
@@ -167,6 +169,13 @@ def blocked_softmax(plan, src, dst, H, Dsrc, scale=1.0):
                                    float(scale), _stream())
     check(st, "ba_blocked_softmax")
     return dst
+
+
+def blocked_softmax_backward(plan, y, dy, dx, H, Dsrc, scale=1.0):
+    st = load().ba_blocked_softmax_backward(plan.ptr, plan._hint(), dtype_code(y.dtype), _ptr(y), _ptr(dy), _ptr(dx),
+                                            H, Dsrc, float(scale), _stream())
+    check(st, "ba_blocked_softmax_backward")
+    return dx
 
 
 def gemm_softmax(plan, A, B, out, H, Dm1, Dm2, Dout, scale=1.0):

@@ -35,6 +35,9 @@ int launch_gemm_f32(const RunArgs &args, const ba_plan_info *info, hipStream_t s
 int launch_softmax(int dtype, void *plan, const void *src, void *dst, int64_t H, int64_t Dsrc, float scale,
                    const ba_plan_info *info, hipStream_t stream);
 
+int launch_softmax_backward(int dtype, void *plan, const void *y, const void *dy, void *dx, int64_t H, int64_t Dsrc,
+                            float scale, const ba_plan_info *info, hipStream_t stream);
+
 // Number of compute units of the current device (cached per device).
 int device_cu_count();
 

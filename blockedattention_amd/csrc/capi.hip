@@ -120,6 +120,16 @@ __attribute__((visibility("default"))) int ba_blocked_softmax(void *plan, const 
     return launch_softmax(dtype, plan, src, dst, H, Dsrc, scale, info, (hipStream_t)stream);
 }
 
+__attribute__((visibility("default"))) int ba_blocked_softmax_backward(void *plan, const ba_plan_info *info,
+                                                                       int dtype, const void *y, const void *dy,
+                                                                       void *dx, int64_t H, int64_t Dsrc,
+                                                                       float scale, ba_stream_t stream) {
+    if (!plan || H < 0 || Dsrc < 0) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dsrc == 0) return BA_OK;
+    if (!y || !dy || !dx) return BA_ERR_INVALID_ARG;
+    return launch_softmax_backward(dtype, plan, y, dy, dx, H, Dsrc, scale, info, (hipStream_t)stream);
+}
+
 __attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_plan_info *info, int dtype,
                                                            const void *A, const void *B, void *out, int out_dtype,
                                                            int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,

@@ -135,4 +135,89 @@ int launch_softmax(int dtype, void *plan, const void *src, void *dst, int64_t H,
     }
 }
 
+// Backward of the blocked softmax: dx = scale * (dy - sum(y * dy)) * y per row
+// (csrc/cuda/spBlkSoftmax.cu:140-180, 271-332; the reference has scale = 1).
+// y is the saved forward output.  Same row mapping as the forward kernel;
+// products and the row sum are fp32 for every dtype.
+struct SoftmaxBwdArgs {
+    void *plan;
+    const void *y;
+    const void *dy;
+    void *dx;
+    int64_t H, Dsrc;
+    float scale;
+};
+
+template <int DT> __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_backward_kernel(SoftmaxBwdArgs a) {
+    typedef typename Io<DT>::T T;
+    PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
+    if (hdr->magic != kPlanMagic || hdr->bad_segments != 0 || hdr->Dout != a.Dsrc) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&hdr->run_errors, 1);
+        return;
+    }
+    const int nseg = hdr->nseg;
+    const PlanView pv = plan_view(a.plan, nseg);
+    const int32_t *pfx = pv.pfx[kPfxRows];
+    const int64_t per_head = hdr->totals[kPfxRows];
+    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int lane = lane_id();
+    const T *ys = reinterpret_cast<const T *>(a.y), *dys = reinterpret_cast<const T *>(a.dy);
+    T *dxs = reinterpret_cast<T *>(a.dx);
+    const int64_t gw = (int64_t)blockIdx.x * kSoftmaxWaves + wave, nw = (int64_t)gridDim.x * kSoftmaxWaves;
+    for (int64_t it = gw; it < per_head * a.H; it += nw) {
+        const int64_t h = it / per_head;
+        const int i = (int)(it - h * per_head);
+        const int g = prefix_search(pfx, nseg, i);
+        const int r = i - pfx[g];
+        const int cols = pv.N[g];
+        const int64_t e0 = h * a.Dsrc + pv.offO[g] + (int64_t)r * cols;
+        const T *y = ys + e0, *dy = dys + e0;
+        T *dx = dxs + e0;
+        if (cols <= 64 * kRegs) {
+            float yv[kRegs], gv[kRegs];
+            float dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < kRegs; ++j) {
+                const int col = lane + 64 * j;
+                yv[j] = (col < cols) ? Io<DT>::ld(y + col) : 0.f;
+                gv[j] = (col < cols) ? Io<DT>::ld(dy + col) : 0.f;
+                dot = fmaf(yv[j], gv[j], dot);
+            }
+            dot = wave_sum(dot);
+#pragma unroll
+            for (int j = 0; j < kRegs; ++j) {
+                const int col = lane + 64 * j;
+                if (col < cols) Io<DT>::st(dx + col, a.scale * (gv[j] - dot) * yv[j]);
+            }
+        } else {
+            float dot = 0.f;
+            for (int col = lane; col < cols; col += 64) dot = fmaf(Io<DT>::ld(y + col), Io<DT>::ld(dy + col), dot);
+            dot = wave_sum(dot);
+            for (int col = lane; col < cols; col += 64)
+                Io<DT>::st(dx + col, a.scale * (Io<DT>::ld(dy + col) - dot) * Io<DT>::ld(y + col));
+        }
+    }
+}
+
+template <int DT>
+static int launch_softmax_bwd_t(const SoftmaxBwdArgs &args, const ba_plan_info *info, hipStream_t stream) {
+    int64_t grid = (int64_t)device_cu_count() * 8;
+    if (info) grid = std::min(grid * 4, (info->total_rows * args.H + kSoftmaxWaves - 1) / kSoftmaxWaves);
+    if (grid <= 0) return BA_OK;
+    hipLaunchKernelGGL(softmax_rows_backward_kernel<DT>, dim3((unsigned)grid), dim3(kSoftmaxThreads), 0, stream,
+                       args);
+    return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+}
+
+int launch_softmax_backward(int dtype, void *plan, const void *y, const void *dy, void *dx, int64_t H, int64_t Dsrc,
+                            float scale, const ba_plan_info *info, hipStream_t stream) {
+    SoftmaxBwdArgs args{plan, y, dy, dx, H, Dsrc, scale};
+    switch (dtype) {
+        case BA_F16: return launch_softmax_bwd_t<BA_F16>(args, info, stream);
+        case BA_BF16: return launch_softmax_bwd_t<BA_BF16>(args, info, stream);
+        case BA_F32: return launch_softmax_bwd_t<BA_F32>(args, info, stream);
+        default: return BA_ERR_UNSUPPORTED;
+    }
+}
+
 }  // namespace ba

@@ -138,6 +138,15 @@ int ba_blocked_softmax(void *plan, const ba_plan_info *info, int dtype, const vo
                        int64_t H, int64_t Dsrc, float scale, ba_stream_t stream);
 
 /*
+ * dx row = scale * (dy row - sum(y row * dy row)) * y row, y being the saved
+ * output of ba_blocked_softmax with the same scale.  Stands in for
+ * sparseBlockedSoftmaxBackwardLaunch (csrc/sparseBlockedAttention.h:21,
+ * csrc/cuda/spBlkSoftmax.cu:418-459).  dx may alias dy.
+ */
+int ba_blocked_softmax_backward(void *plan, const ba_plan_info *info, int dtype, const void *y, const void *dy,
+                                void *dx, int64_t H, int64_t Dsrc, float scale, ba_stream_t stream);
+
+/*
  * Fused pair: out = softmax(scale * A_g B_g^T) per segment with the scores kept
  * in fp32 registers between the two steps.  Equivalent to ba_varlen_gemm
  * followed by ba_blocked_softmax on (M, N, accumOut) without the intermediate

@@ -139,6 +139,18 @@ def blocked_softmax(src, rows, cols, scale=1.0, accum=None):
     return out
 
 
+def blocked_softmax_backward(y, dy, rows, cols, scale=1.0):
+    y, py = _f32(y); dy, pdy = _f32(dy)
+    rows, pr = _i64(rows); cols, pc = _i64(cols)
+    acc = softmax_accum(rows, cols)
+    H, D = y.shape
+    dx = np.empty_like(y)
+    c = ctypes.c_int64
+    lib().oracle_blocked_softmax_backward_f32(py, pdy, dx.ctypes.data_as(_F32P), c(H), c(D), c(rows.shape[0]),
+                                              acc.ctypes.data_as(_I64P), pr, pc, ctypes.c_float(scale))
+    return dx
+
+
 def gemm_softmax(A, Bm, M, N, K, scale=1.0, return_scores=False):
     A, pA = _f32(A); Bm, pB = _f32(Bm)
     M, pM = _i64(M); N, pN = _i64(N); K, pK = _i64(K)

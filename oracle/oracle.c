@@ -259,6 +259,27 @@ ORACLE_API void oracle_blocked_softmax_f32(const float *src, float *out, int64_t
 }
 
 /*
+ * Softmax backward: dx = scale * (dy - sum_c(y*dy)) * y per row, y the forward
+ * output (csrc/cuda/spBlkSoftmax.cu:140-180; the reference has scale = 1).
+ * Evaluated in double and rounded to float once.
+ */
+ORACLE_API void oracle_blocked_softmax_backward_f32(const float *y, const float *dy, float *dx, int64_t H,
+                                                    int64_t Dsrc, int64_t nseg, const int64_t *accum,
+                                                    const int64_t *rows, const int64_t *cols, float scale) {
+    for (int64_t h = 0; h < H; ++h)
+        for (int64_t g = 0; g < nseg; ++g) {
+            const int64_t nc = cols[g];
+            for (int64_t r = 0; r < rows[g]; ++r) {
+                const int64_t e0 = h * Dsrc + accum[g] + r * nc;
+                double dot = 0.0;
+                for (int64_t c = 0; c < nc; ++c) dot += (double)y[e0 + c] * (double)dy[e0 + c];
+                for (int64_t c = 0; c < nc; ++c)
+                    dx[e0 + c] = (float)((double)scale * ((double)dy[e0 + c] - dot) * (double)y[e0 + c]);
+            }
+        }
+}
+
+/*
  * The pair the benchmark names: softmax(scale * A_g B_g^T) per segment, the
  * scores kept in float between the two steps (no 16-bit rounding), i.e.
  * oracle_varlen_gemm_f32 followed by oracle_blocked_softmax_f32 with

@@ -1,0 +1,75 @@
+"""Fused GEMM + softmax through the C ABI: every width class, fp32 output, the
+large configuration at full size through size-independent properties."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blockedattention_amd import capi, workloads
+from _util import assert_probs_close, make_plan, random_operands, run_all
+
+pytestmark = pytest.mark.gpu
+
+
+def test_split_and_wide_rows(dev):
+    # 256 < N <= 4096: one workgroup per strip; N > 4096: two sweeps.
+    M = [20, 3, 33, 16, 5]; N = [257, 4096, 1000, 4097, 9001]; K = [64, 128, 32, 72, 8]
+    plan = run_all(dev, M, N, K, 2, torch.float16, 0.2, check_gemm=False)
+    assert plan.info.split_items == 2 + 1 + 3 and plan.info.wide_items == 1 + 1
+    run_all(dev, M, N, K, 2, torch.bfloat16, 0.1, seed=1, check_gemm=False)
+
+
+def test_negative_and_zero_scale(dev):
+    M = [9, 30, 4]; N = [300, 17, 5000]; K = [16, 64, 8]
+    for scale in (-0.3, 0.0):
+        run_all(dev, M, N, K, 2, torch.float16, scale, check_gemm=False)
+
+
+def test_fp32_probabilities(dev):
+    w = workloads.make(3)
+    M, N, K = w.M[:200], w.N[:200], w.K[:200]
+    A, B = random_operands(M, N, K, 2, torch.bfloat16)
+    plan = make_plan(dev, M, N, K)
+    i = plan.info
+    out = torch.full((2, i.Dout), float("nan"), dtype=torch.float32, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, 2, i.Dm1, i.Dm2, i.Dout, w.scale)
+    ref = oracle.per_segment_torch(A, B, M, N, K, w.scale)
+    assert (out.cpu() - ref).abs().max().item() <= 2e-5        # fp32 output: the 1e-3 bound holds with room
+
+
+def test_large_segments_one_head_against_oracle(dev):
+    # Configuration 5 shape (n in [1024, 4096], K = 128, bf16) on its three smallest segments.
+    w = workloads.make(5)
+    idx = np.argsort(w.M)[:3]
+    M = w.M[idx]
+    A, B = random_operands(M, M, [128] * 3, 1, torch.bfloat16, sigma=w.sigma)
+    plan = make_plan(dev, M, M, [128] * 3)
+    i = plan.info
+    out = torch.empty((1, i.Dout), dtype=torch.bfloat16, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, 1, i.Dm1, i.Dm2, i.Dout, w.scale)
+    assert_probs_close(out, oracle.per_segment_torch(A, B, M, M, [128] * 3, w.scale), "cfg5 subset")
+
+
+def test_config5_full_size_properties(dev):
+    # 16 segments x 16 heads, 1.93e9 probabilities: rows sum to one, and sampled rows match the oracle.
+    w = workloads.make(5)
+    A, B = w.operands()
+    plan = make_plan(dev, w.M, w.N, w.K)
+    Ad, Bd = A.to(dev), B.to(dev)
+    out = torch.empty((w.heads, w.Dout), dtype=torch.bfloat16, device=dev)
+    capi.gemm_softmax(plan, Ad, Bd, out, w.heads, w.Dm1, w.Dm2, w.Dout, w.scale)
+    a1, a2, ao = oracle.lists_to_accum(w.M, w.N, w.K)
+    rng = np.random.default_rng(0)
+    for g in range(w.nseg):
+        n = int(w.M[g])
+        blk = out[:, ao[g]:ao[g + 1]].reshape(w.heads, n, n)
+        sums = blk.float().sum(-1)
+        assert (sums - 1).abs().max().item() < 2e-2, g          # bf16 rounding of n values of ~1/n
+        h = int(rng.integers(0, w.heads)); r = int(rng.integers(0, n))
+        a = A[h, a1[g] + r * 128:a1[g] + (r + 1) * 128].float()
+        b = B[h, a2[g]:a2[g + 1]].float().reshape(n, 128)
+        ref = torch.softmax((b @ a) * w.scale, -1)
+        got = blk[h, r].float().cpu()
+        assert ((got - ref).abs() <= 1e-3 + ref * 2.0 ** -8).all(), (g, h, r)
+        assert ((got - ref.bfloat16().float()).abs() <= ref * 2.0 ** -7 + 1e-9).all(), (g, h, r)
+    assert plan.read().run_errors == 0

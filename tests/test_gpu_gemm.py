@@ -1,0 +1,144 @@
+"""Varlen GEMM through the C ABI against the oracle (scores within rel 1e-2)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blockedattention_amd import capi, workloads
+from _util import assert_scores_close, make_plan, random_operands, run_all
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4])
+def test_benchmark_configs(dev, cfg):
+    w = workloads.make(cfg)
+    run_all(dev, w.M, w.N, w.K, w.heads, w.dtype, w.scale, dist=w.dist, sigma=w.sigma)
+
+
+def test_integer_closed_form_11_13_5(dev):
+    # csrc/sparseBlockedAttention.cpp:216-241; values are exact in fp16 products and fp32 sums,
+    # results up to 19630 are not all fp16-representable, so compare after the one rounding.
+    A = torch.arange(55, dtype=torch.float32).reshape(1, 55)
+    B = torch.arange(65, dtype=torch.float32).reshape(1, 65)
+    expect = torch.tensor([[sum((5 * r + t) * (5 * c + t) for t in range(5)) for c in range(13)] for r in range(11)],
+                          dtype=torch.float32).reshape(1, -1)
+    plan = make_plan(dev, [11], [13], [5])
+    assert plan.info.slow_items == 1                 # K = 5: element-wise path
+    for dtype in (torch.float16, torch.float32):
+        out = torch.empty((1, 143), dtype=dtype, device=dev)
+        capi.varlen_gemm(plan, A.to(dtype).to(dev), B.to(dtype).to(dev), out, 1, 55, 65, 143)
+        assert torch.equal(out.cpu(), expect.to(dtype))
+
+
+def test_reference_profile_shapes_fp32(dev):
+    # test/pytest.py:7-19: H=128, (33,33,64), (99,99,64), (64,64,64), fp32, lists only.
+    M = [33, 99, 64]; K = [64] * 3
+    A, B = random_operands(M, M, K, 128, torch.float32, seed=1)
+    plan = make_plan(dev, M, M, K)
+    out = torch.empty((128, plan.info.Dout), dtype=torch.float32, device=dev)
+    capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, 128, plan.info.Dm1, plan.info.Dm2, plan.info.Dout)
+    ref = oracle.per_segment_torch(A, B, M, M, K, want="scores")
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_odd_k_61_half_from_prefix_sums(dev):
+    # csrc/sparseBlockedAttention.cpp:170-192: H=128, (33,33,61) + (127,127,61), half, prefix sums only.
+    M = np.array([33, 127]); K = np.array([61, 61]); H = 128
+    a1, a2, ao = [torch.as_tensor(a).to(dev) for a in oracle.lists_to_accum(M, M, K)]
+    plan = capi.plan_gemm(2, dev, None, None, None, a1, a2, ao, mode=capi.META_FROM_ACCUM)
+    info = plan.read()
+    assert info.slow_items == 3 + 8 and info.gemm_items == 0
+    A, B = random_operands(M, M, K, H, torch.float16, seed=2)
+    out = torch.empty((H, info.Dout), dtype=torch.float16, device=dev)
+    capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, H, info.Dm1, info.Dm2, info.Dout)
+    assert_scores_close(out, oracle.per_segment_torch(A, B, M, M, K, want="scores"), "K=61")
+    fused = torch.empty_like(out)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), fused, H, info.Dm1, info.Dm2, info.Dout, 0.125)
+    torch.testing.assert_close(fused.float().cpu(), oracle.per_segment_torch(A, B, M, M, K, 0.125), rtol=0, atol=1e-3)
+
+
+def test_legacy_square_graphs(dev):
+    # csrc/sparseBlockedAttention.cpp:147-151: n = {10,5,20,5,60}, d = 32, H = 8.
+    n = [10, 5, 20, 5, 60]
+    run_all(dev, n, n, [32] * 5, 8, torch.float16, 32 ** -0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("t1,t2", [(True, False), (False, True), (True, True)])
+def test_transposed_layouts(dev, dtype, t1, t2):
+    rng = np.random.default_rng(11)
+    M = rng.integers(1, 70, 9); N = rng.integers(1, 300, 9); K = rng.choice([8, 24, 64, 5], 9); H = 3
+    A, B = random_operands(M, N, K, H, dtype, seed=3)
+    plan = make_plan(dev, M, N, K)
+    out = torch.full((H, plan.info.Dout), float("nan"), dtype=dtype, device=dev)
+    capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, H, plan.info.Dm1, plan.info.Dm2, plan.info.Dout, t1, t2)
+    ref = oracle.varlen_gemm(A.float().numpy(), B.float().numpy(), M, N, K, t1, t2, f64acc=True)
+    assert_scores_close(out, torch.from_numpy(ref), f"transpose {t1} {t2}")
+
+
+def test_ragged_edges_and_degenerate_segments(dev):
+    # rows/cols not multiples of 16, N across the 256-column chunk boundary, K % 32 in {8,16,24},
+    # K = 0 (zeros), M = 0 and N = 0 (no work), odd N (unaligned row starts in the output).
+    M = [1, 17, 16, 31, 5, 0, 7, 40, 3]; N = [1, 255, 257, 513, 33, 9, 0, 300, 1031]; K = [8, 16, 24, 40, 0, 8, 8, 72, 96]
+    run_all(dev, M, N, K, 2, torch.float16, 0.2, check_softmax=False)
+    run_all(dev, M, N, K, 3, torch.bfloat16, 0.2, check_softmax=False)
+
+
+def test_unaligned_base_pointers_and_odd_head_stride(dev):
+    M = np.array([20, 9]); N = np.array([18, 40]); K = np.array([8, 16]); H = 2
+    A, B = random_operands(M, N, K, H, torch.float16, seed=5)
+    plan = make_plan(dev, M, N, K)
+    i = plan.info
+    ref = oracle.per_segment_torch(A, B, M, N, K, want="scores")
+    big = torch.zeros(H * i.Dm1 + 1, dtype=torch.float16, device=dev)
+    big[1:] = A.reshape(-1).to(dev)                            # base pointer 2 bytes off
+    out = torch.empty((H, i.Dout), dtype=torch.float16, device=dev)
+    capi.varlen_gemm(plan, big[1:], B.to(dev), out, H, i.Dm1, i.Dm2, i.Dout)
+    assert_scores_close(out, ref, "unaligned A")
+    # an aligned segment followed by K = 4 with odd M: the per-head stride (60) is not a multiple
+    # of 8 elements, so heads 1 and 2 start unaligned and no segment may use 16-byte loads
+    M2, N2, K2 = [6, 3], [10, 5], [8, 4]
+    A2, B2 = random_operands(M2, N2, K2, 3, torch.bfloat16, seed=6)
+    plan2 = make_plan(dev, M2, N2, K2)
+    assert (plan2.info.Dm1, plan2.info.Dm2, plan2.info.Dout, plan2.info.gemm_items) == (60, 100, 75, 1)
+    out2 = torch.empty((3, 75), dtype=torch.bfloat16, device=dev)
+    capi.varlen_gemm(plan2, A2.to(dev), B2.to(dev), out2, 3, 60, 100, 75)
+    assert_scores_close(out2, oracle.per_segment_torch(A2, B2, M2, N2, K2, want="scores"), "odd head stride")
+
+
+def test_gapped_prefix_sums_given_with_lists(dev):
+    M, N, K = [4, 20], [6, 33], [8, 16]
+    a1 = [0, 40, 40 + 320]; a2 = [0, 56, 56 + 528]; ao = [0, 30, 30 + 660]      # gaps of 8, 8 and 6 elements
+    d = lambda x: torch.as_tensor(np.asarray(x, np.int64)).to(dev)
+    plan = capi.plan_gemm(2, dev, d(M), d(N), d(K), d(a1), d(a2), d(ao), mode=capi.META_GIVEN)
+    info = plan.read()
+    assert (info.Dm1, info.Dm2, info.Dout) == (360, 584, 690)
+    g = torch.Generator().manual_seed(0)
+    A = torch.randn((2, 360), generator=g).half(); B = torch.randn((2, 584), generator=g).half()
+    out = torch.full((2, 690), 9.0, dtype=torch.float16, device=dev)
+    capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, 2, 360, 584, 690)
+    o = out.float().cpu()
+    for m, n, k, o1, o2, oo in zip(M, N, K, a1, a2, ao):
+        ref = A[:, o1:o1 + m * k].float().reshape(2, m, k) @ B[:, o2:o2 + n * k].float().reshape(2, n, k).transpose(1, 2)
+        assert_scores_close(o[:, oo:oo + m * n], ref.reshape(2, -1), "gapped")
+    assert (o[:, 24:30] == 9.0).all()                          # the gap is never written
+
+
+def test_many_tiny_segments_are_packed(dev):
+    rng = np.random.default_rng(13)
+    n = rng.integers(1, 9, 400)
+    plan = run_all(dev, n, n, [64] * 400, 4, torch.float16, 0.125)
+    assert plan.info.pack_items > 100
+    m = rng.integers(1, 6, 300); nn = rng.integers(1, 6, 300)      # non-square tiny segments, bf16, K = 128
+    plan = run_all(dev, m, nn, [128] * 300, 2, torch.bfloat16, 128 ** -0.5)
+    assert plan.info.pack_items > 50
+
+
+def test_unsupported_dtype_and_empty_calls(dev):
+    plan = make_plan(dev, [4], [4], [8])
+    x = torch.zeros((1, 32), dtype=torch.float64, device=dev)
+    with pytest.raises(capi.BlockedAttentionError, match="unsupported dtype"):
+        capi.varlen_gemm(plan, x, x, x, 1, 32, 32, 16)
+    e = torch.empty((0, 32), dtype=torch.float16, device=dev)
+    capi.varlen_gemm(plan, e, e, torch.empty((0, 16), dtype=torch.float16, device=dev), 0, 32, 32, 16)

@@ -1,0 +1,149 @@
+"""Device-side scheduler against the oracle: offsets and lists bit-exact, work
+items an exact cover, bad metadata rejected (all through the C ABI)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blockedattention_amd import capi, workloads
+from _util import dev_i64, make_plan
+
+pytestmark = pytest.mark.gpu
+
+
+def expected_items(M, N, K):
+    """Host restatement of the plan's classification for lists-only metadata."""
+    M = np.asarray(M); N = np.asarray(N); K = np.asarray(K)
+    a1, a2, _ = oracle.lists_to_accum(M, N, K)
+    aligned = ((K | a1[:-1] | a2[:-1]) & 7) == 0
+    strips = np.where(N >= 1, -(-M // 16), 0)
+    pack = np.zeros(len(M), np.int64)
+    for w0 in range(0, len(M), 16):
+        i = w0
+        end = min(w0 + 16, len(M))
+        while i < end:
+            ln = sm = sn = 0
+            while i + ln < end:
+                g = i + ln
+                if M[g] < 1 or N[g] < 1 or not aligned[g] or K[g] != K[i] or K[i] < 1 or not aligned[i]:
+                    break
+                if sm + M[g] > 16 or sn + N[g] > 16:
+                    break
+                sm += M[g]; sn += N[g]; ln += 1
+            if ln >= 2:
+                pack[i] = ln; pack[i + 1:i + ln] = -1; i += ln
+            else:
+                i += 1
+    ok = aligned & (pack == 0)
+    return {
+        "gemm_items": int((strips * -(-N // 256))[ok].sum()),
+        "strip_items": int(strips[ok & (N <= 256)].sum()),
+        "split_items": int(strips[ok & (N > 256) & (N <= 4096)].sum()),
+        "wide_items": int(strips[ok & (N > 4096)].sum()),
+        "pack_items": int((pack > 0).sum()),
+        "slow_items": int(strips[~aligned].sum()),
+        "total_rows": int(M[N >= 1].sum()),
+    }
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_offsets_bit_exact_and_items_cover(dev, cfg):
+    w = workloads.make(cfg)
+    plan = make_plan(dev, w.M, w.N, w.K)
+    a1, a2, ao = oracle.lists_to_accum(w.M, w.N, w.K)
+    for got, ref in zip(plan.keep[3:], (a1, a2, ao)):
+        assert got.dtype == torch.int64 and np.array_equal(got.cpu().numpy(), ref)
+    info = plan.info.as_dict()
+    assert (info["Dm1"], info["Dm2"], info["Dout"]) == (w.Dm1, w.Dm2, w.Dout)
+    assert (info["max_M"], info["max_N"], info["max_K"]) == (w.M.max(), w.N.max(), w.K.max())
+    for k, v in expected_items(w.M, w.N, w.K).items():
+        assert info[k] == v, (k, info[k], v)
+    assert info["bad_segments"] == 0
+
+
+@pytest.mark.parametrize("cfg", [1, 3, 4, 5])
+def test_lists_from_prefix_sums_are_exact(dev, cfg):
+    w = workloads.make(cfg)
+    a1, a2, ao = [dev_i64(a, dev) for a in oracle.lists_to_accum(w.M, w.N, w.K)]
+    M = torch.full((w.nseg,), -7, dtype=torch.int64, device=dev); N = M.clone(); K = M.clone()
+    plan = capi.plan_gemm(w.nseg, dev, M, N, K, a1, a2, ao, mode=capi.META_FROM_ACCUM)
+    info = plan.read()
+    assert np.array_equal(M.cpu().numpy(), w.M) and np.array_equal(N.cpu().numpy(), w.N)
+    assert np.array_equal(K.cpu().numpy(), w.K)
+    assert (info.Dm1, info.Dm2, info.Dout, info.bad_segments) == (w.Dm1, w.Dm2, w.Dout, 0)
+
+
+def test_lists_from_prefix_sums_large_and_degenerate(dev):
+    M = np.array([4097, 99991, 16777217, 3, 0, 1 << 20]); N = np.array([4095, 7, 3, 16777219, 0, 1 << 20])
+    K = np.array([127, 99989, 5, 2, 0, 1 << 20])
+    a = [dev_i64(x, dev) for x in oracle.lists_to_accum(M, N, K)]
+    m = torch.empty(6, dtype=torch.int64, device=dev); n = m.clone(); k = m.clone()
+    info = capi.plan_gemm(6, dev, m, n, k, *a, mode=capi.META_FROM_ACCUM).read()
+    assert info.bad_segments == 0
+    assert np.array_equal(m.cpu().numpy(), M) and np.array_equal(n.cpu().numpy(), N) and np.array_equal(k.cpu().numpy(), K)
+    # inconsistent areas are rejected, and reported as -1 like the oracle does
+    a1, a2, ao = dev_i64([0, 6, 12], dev), dev_i64([0, 10, 20], dev), dev_i64([0, 14, 29], dev)
+    m = torch.empty(2, dtype=torch.int64, device=dev); n = m.clone(); k = m.clone()
+    plan = capi.plan_gemm(2, dev, m, n, k, a1, a2, ao, mode=capi.META_FROM_ACCUM)
+    info = plan.read(raise_on_bad=False)
+    om, on, ok, obad = oracle.accum_to_lists([0, 6, 12], [0, 10, 20], [0, 14, 29])
+    assert info.bad_segments == obad == 1
+    assert np.array_equal(m.cpu().numpy(), om) and np.array_equal(k.cpu().numpy(), ok)
+
+
+def test_more_segments_than_one_scheduler_pass(dev):
+    rng = np.random.default_rng(7)
+    B = 5000
+    M = rng.integers(0, 40, B); N = rng.integers(0, 40, B); K = rng.choice([0, 8, 16, 24, 61], B)
+    plan = make_plan(dev, M, N, K)
+    a1, a2, ao = oracle.lists_to_accum(M, N, K)
+    for got, ref in zip(plan.keep[3:], (a1, a2, ao)):
+        assert np.array_equal(got.cpu().numpy(), ref)
+    info = plan.info.as_dict()
+    for k, v in expected_items(M, N, K).items():
+        assert info[k] == v, (k, info[k], v)
+
+
+def test_bad_metadata_is_rejected_and_kernels_refuse_to_run(dev):
+    M = dev_i64([4, -1, 3], dev); N = dev_i64([4, 2, 3], dev); K = dev_i64([8, 8, 8], dev)
+    plan = capi.plan_gemm(3, dev, M, N, K, mode=capi.META_FROM_LISTS)
+    with pytest.raises(capi.BlockedAttentionError, match="metadata"):
+        plan.read()
+    info = plan.read(raise_on_bad=False)
+    assert info.bad_segments == 1
+    # given both halves, a prefix sum too small for its segment is rejected
+    a1 = dev_i64([0, 32, 40], dev); a2 = dev_i64([0, 32, 64], dev); ao = dev_i64([0, 16, 32], dev)
+    plan = capi.plan_gemm(2, dev, dev_i64([4, 4], dev), dev_i64([4, 4], dev), dev_i64([8, 8], dev), a1, a2, ao,
+                          mode=capi.META_GIVEN)
+    assert plan.read(raise_on_bad=False).bad_segments == 1
+    out = torch.full((1, 32), 7.0, dtype=torch.float16, device=dev)
+    A = torch.zeros((1, 40), dtype=torch.float16, device=dev); B = torch.zeros((1, 64), dtype=torch.float16, device=dev)
+    capi.varlen_gemm(plan, A, B, out, 1, 40, 64, 32)
+    torch.cuda.synchronize()
+    assert (out == 7.0).all() and plan.read(raise_on_bad=False).run_errors == 1
+
+
+def test_size_mismatch_makes_kernels_refuse(dev):
+    plan = make_plan(dev, [4], [4], [8])
+    out = torch.full((1, 16), 7.0, dtype=torch.float16, device=dev)
+    A = torch.zeros((1, 64), dtype=torch.float16, device=dev)
+    capi.varlen_gemm(plan, A, A, out, 1, 64, 64, 16)       # Dm1 should be 32
+    torch.cuda.synchronize()
+    assert (out == 7.0).all() and plan.read(raise_on_bad=False).run_errors == 1
+
+
+def test_softmax_plan_offsets(dev):
+    rows = [33, 99, 64, 0, 5]; cols = [64, 64, 64, 7, 0]
+    acc = torch.empty(6, dtype=torch.int64, device=dev)
+    plan = capi.plan_softmax(5, dev, dev_i64(rows, dev), dev_i64(cols, dev), acc)
+    info = plan.read()
+    assert np.array_equal(acc.cpu().numpy(), oracle.softmax_accum(rows, cols))
+    assert info.Dout == 12544 and info.total_rows == 196
+
+
+def test_empty_batch(dev):
+    e = torch.empty(0, dtype=torch.int64, device=dev)
+    a = [torch.full((1,), -1, dtype=torch.int64, device=dev) for _ in range(3)]
+    info = capi.plan_gemm(0, dev, e, e, e, *a, mode=capi.META_FROM_LISTS).read()
+    assert (info.nseg, info.Dm1, info.Dm2, info.Dout, info.gemm_items) == (0, 0, 0, 0, 0)
+    assert all(int(t[0]) == 0 for t in a)

@@ -1,0 +1,119 @@
+"""Pins the oracle's integer side (offsets, list derivation, work-lists) on the CPU.
+
+Checks are chosen so that a plausible mistake fails one of them: a dropped
+leading zero or an inclusive scan fails the numpy comparison and the published
+totals; swapped M/N or N/K in a product fails the non-square configuration 4;
+a float square root fails the large-size round trips; a work-list that skips
+or repeats a tile fails the exact-cover brute force.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from blockedattention_amd import workloads
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "seed0_totals.json")))
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_prefix_sums_match_published_totals_and_numpy(cfg):
+    w = workloads.make(cfg)
+    g = GOLD[f"cfg{cfg}"]
+    assert w.nseg == g["segments"] and w.heads == g["heads"] and int(w.M.sum()) == g["rows"]
+    a1, a2, ao = oracle.lists_to_accum(w.M, w.N, w.K)
+    assert (int(a1[-1]), int(a2[-1]), int(ao[-1])) == (g["Dm1"], g["Dm2"], g["Dout"])
+    for acc, prod in ((a1, w.M * w.K), (a2, w.N * w.K), (ao, w.M * w.N)):
+        assert acc.dtype == np.int64 and acc.shape == (w.nseg + 1,)
+        assert np.array_equal(acc, np.concatenate([[0], np.cumsum(prod)]))
+    if cfg == 5:
+        assert [int(v) for v in w.M] == g["n"]
+
+
+def test_softmax_accum_is_rows_times_cols():
+    rows = np.array([33, 99, 64, 0, 5]); cols = np.array([64, 64, 64, 7, 0])
+    assert np.array_equal(oracle.softmax_accum(rows, cols), [0, 2112, 8448, 12544, 12544, 12544])
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_accum_to_lists_round_trip(cfg):
+    w = workloads.make(cfg)
+    M, N, K, bad = oracle.accum_to_lists(*oracle.lists_to_accum(w.M, w.N, w.K))
+    assert bad == 0
+    assert np.array_equal(M, w.M) and np.array_equal(N, w.N) and np.array_equal(K, w.K)
+
+
+def test_accum_to_lists_brute_force_small():
+    r = np.arange(1, 41)
+    M, N, K = [a.ravel() for a in np.meshgrid(r, r, r, indexing="ij")]
+    m, n, k, bad = oracle.accum_to_lists(*oracle.lists_to_accum(M, N, K))
+    assert bad == 0 and np.array_equal(m, M) and np.array_equal(n, N) and np.array_equal(k, K)
+
+
+def test_accum_to_lists_large_sizes_exact():
+    # float32 sqrt/division (the reference's route) is off by one here; exact integers are not.
+    M = np.array([4097, 99991, 16777217, 3, 1 << 20]); N = np.array([4095, 7, 3, 16777219, 1 << 20])
+    K = np.array([127, 99989, 5, 2, 1 << 20])
+    m, n, k, bad = oracle.accum_to_lists(*oracle.lists_to_accum(M, N, K))
+    assert bad == 0 and np.array_equal(m, M) and np.array_equal(n, N) and np.array_equal(k, K)
+
+
+def test_accum_to_lists_zero_and_inconsistent_segments():
+    a1 = np.array([0, 0, 6, 6]); a2 = np.array([0, 0, 10, 13]); ao = np.array([0, 0, 15, 15])
+    # segment 0: all areas zero -> (0,0,0); segment 1: (3,5,2); segment 2: mk=0, nk=3, mn=0 -> inconsistent
+    m, n, k, bad = oracle.accum_to_lists(a1, a2, ao)
+    assert bad == 1
+    assert (m[0], n[0], k[0]) == (0, 0, 0) and (m[1], n[1], k[1]) == (3, 5, 2) and m[2] == -1
+    # areas that match no integer triple
+    _, _, _, bad = oracle.accum_to_lists([0, 6], [0, 10], [0, 14])
+    assert bad == 1
+
+
+def test_reference_tile_choice_on_the_five_configs():
+    # Global tile the reference's heuristic picks per configuration (BM = BN).
+    expect = {1: 32, 2: 128, 3: 64, 4: 128, 5: 128}
+    for cfg, tile in expect.items():
+        w = workloads.make(cfg)
+        bm, bn, bk = oracle.ref_tile_choice(w.M, w.N, half_like=True)
+        assert (bm, bn) == (tile, tile), (cfg, bm, bn)
+        assert bk in (8, 16, 32)
+
+
+def test_reference_tile_counts():
+    # Tiles per head at 128x128 and at 32x32, per configuration.
+    at128 = {2: 256, 3: 1365, 4: 1262, 5: 7700}
+    at32 = {1: 64, 2: 2562, 3: 7768}
+    for cfg, n in at128.items():
+        w = workloads.make(cfg)
+        assert oracle.gemm_worklist(w.M, w.N, 128, 128).shape[0] == n
+    for cfg, n in at32.items():
+        w = workloads.make(cfg)
+        assert oracle.gemm_worklist(w.M, w.N, 32, 32).shape[0] == n
+
+
+@pytest.mark.parametrize("bm,bn", [(32, 32), (64, 128), (16, 256)])
+def test_gemm_worklist_covers_every_output_exactly_once(bm, bn):
+    rng = np.random.default_rng(3)
+    M = rng.integers(0, 150, 23); N = rng.integers(0, 300, 23)
+    wl = oracle.gemm_worklist(M, N, bm, bn)
+    assert wl.shape[0] == int((-(-M // bm) * -(-N // bn)).sum())
+    for g in range(len(M)):
+        cover = np.zeros((M[g], N[g]), np.int32)
+        ntile = -(-N[g] // bn)
+        for seg, t in wl[wl[:, 0] == g]:
+            r0, c0 = (t // ntile) * bm, (t % ntile) * bn
+            assert r0 < M[g] and c0 < N[g]
+            cover[r0:r0 + bm, c0:c0 + bn] += 1
+        assert (cover == 1).all()
+    assert np.array_equal(wl[:, 0], np.sort(wl[:, 0]))     # segment-major
+
+
+def test_softmax_worklist_is_a_bijection_onto_rows():
+    rows = np.array([3, 0, 5, 1])
+    wl = oracle.softmax_worklist(rows)
+    assert wl.tolist() == [[0, 0], [0, 1], [0, 2], [2, 0], [2, 1], [2, 2], [2, 3], [2, 4], [3, 0]]
+    w = workloads.make(3)
+    wl = oracle.softmax_worklist(w.M)
+    assert wl.shape[0] == GOLD["cfg3"]["rows"] and len({(int(a), int(b)) for a, b in wl}) == wl.shape[0]

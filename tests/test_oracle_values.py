@@ -1,0 +1,132 @@
+"""Pins the oracle's floating-point side on the CPU against closed forms and libraries.
+
+GEMM: the integer closed form of the reference's arange case (11,13,5)
+(a transposed operand, a wrong stride or a dropped k term changes it), identity
+operands, dense batched matmul for equal-sized segments, numpy per segment for
+both transposed layouts.  Softmax: scipy.special.softmax, rows summing to one,
+constant rows, shift invariance, all -inf rows.  Backward: torch.autograd.
+The two independent statements (C loops, per-segment torch) must agree.
+"""
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+import oracle
+from blockedattention_amd import workloads
+
+
+def test_gemm_integer_closed_form_11_13_5():
+    # csrc/sparseBlockedAttention.cpp:216-241: H=1, (M,N,K)=(11,13,5), inputs arange.
+    A = np.arange(55, dtype=np.float32)[None]
+    B = np.arange(65, dtype=np.float32)[None]
+    out = oracle.varlen_gemm(A, B, [11], [13], [5])
+    expect = np.array([[sum((5 * r + t) * (5 * c + t) for t in range(5)) for c in range(13)] for r in range(11)])
+    assert np.array_equal(out.reshape(11, 13), expect.astype(np.float32))
+
+
+def test_gemm_identity_operand_reproduces_a():
+    rng = np.random.default_rng(0)
+    M, K = np.array([7, 3]), np.array([5, 9])
+    A = rng.standard_normal((2, int((M * K).sum()))).astype(np.float32)
+    eye = np.concatenate([np.eye(5).ravel(), np.eye(9).ravel()]).astype(np.float32)
+    out = oracle.varlen_gemm(A, np.stack([eye, eye]), M, K, K)     # N = K, B = I
+    assert np.array_equal(out, A)
+
+
+def test_gemm_equal_segments_match_dense_bmm():
+    rng = np.random.default_rng(1)
+    H, B, n, K = 3, 6, 10, 16
+    A = rng.standard_normal((H, B * n * K)).astype(np.float32)
+    Bm = rng.standard_normal((H, B * n * K)).astype(np.float32)
+    out = oracle.varlen_gemm(A, Bm, [n] * B, [n] * B, [K] * B, f64acc=True)
+    dense = np.einsum("hbik,hbjk->hbij", A.reshape(H, B, n, K).astype(np.float64),
+                      Bm.reshape(H, B, n, K).astype(np.float64))
+    np.testing.assert_allclose(out, dense.reshape(H, -1).astype(np.float32), rtol=1e-6, atol=1e-6)
+    out32 = oracle.varlen_gemm(A, Bm, [n] * B, [n] * B, [K] * B)
+    np.testing.assert_allclose(out32, out, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("t1,t2", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_transposed_layouts_match_numpy(t1, t2):
+    rng = np.random.default_rng(2)
+    M, N, K = np.array([5, 8, 1]), np.array([4, 3, 6]), np.array([7, 2, 9])
+    H = 2
+    A = rng.standard_normal((H, int((M * K).sum()))).astype(np.float32)
+    Bm = rng.standard_normal((H, int((N * K).sum()))).astype(np.float32)
+    out = oracle.varlen_gemm(A, Bm, M, N, K, transpose1=t1, transpose2=t2, f64acc=True)
+    o1 = o2 = oo = 0
+    for m, n, k in zip(M, N, K):
+        a = A[:, o1:o1 + m * k].reshape(H, k, m).transpose(0, 2, 1) if t1 else A[:, o1:o1 + m * k].reshape(H, m, k)
+        b = Bm[:, o2:o2 + n * k].reshape(H, k, n).transpose(0, 2, 1) if t2 else Bm[:, o2:o2 + n * k].reshape(H, n, k)
+        ref = np.einsum("hik,hjk->hij", a.astype(np.float64), b.astype(np.float64)).reshape(H, -1)
+        np.testing.assert_allclose(out[:, oo:oo + m * n], ref, rtol=1e-6, atol=1e-6)
+        o1 += m * k; o2 += n * k; oo += m * n
+
+
+def test_gemm_zero_k_and_empty_segments():
+    # segment 0 has K = 0 (2x3 zeros), segment 1 has no rows, segment 2 has no columns
+    out = oracle.varlen_gemm(np.ones((1, 21), np.float32), np.ones((1, 20), np.float32), [2, 0, 3], [3, 4, 0], [0, 5, 7])
+    assert out.shape == (1, 6) and np.array_equal(out, np.zeros((1, 6), np.float32))
+
+
+def test_softmax_matches_scipy_and_invariants():
+    rng = np.random.default_rng(4)
+    rows, cols = np.array([33, 99, 64, 2]), np.array([64, 64, 64, 2047])   # reference check shapes + a long row
+    H = 3
+    src = (rng.standard_normal((H, int((rows * cols).sum()))) * 3).astype(np.float32)
+    for scale in (1.0, 0.125, -0.5):
+        out = oracle.blocked_softmax(src, rows, cols, scale)
+        o = 0
+        for r, c in zip(rows, cols):
+            blk = src[:, o:o + r * c].reshape(H, r, c).astype(np.float64) * scale
+            np.testing.assert_allclose(out[:, o:o + r * c].reshape(H, r, c), scipy.special.softmax(blk, axis=-1),
+                                       rtol=2e-6, atol=1e-9)
+            np.testing.assert_allclose(out[:, o:o + r * c].reshape(H, r, c).sum(-1), 1.0, rtol=1e-5)
+            o += r * c
+    shifted = oracle.blocked_softmax(src + 11.0, rows, cols)
+    np.testing.assert_allclose(shifted, oracle.blocked_softmax(src, rows, cols), rtol=1e-4, atol=1e-7)
+
+
+def test_softmax_constant_and_all_neg_inf_rows():
+    out = oracle.blocked_softmax(np.full((1, 12), 3.5, np.float32), [2], [6])
+    np.testing.assert_allclose(out, 1.0 / 6.0, rtol=1e-7)
+    x = np.array([[-np.inf, -np.inf, 0.0, -np.inf]], np.float32)
+    out = oracle.blocked_softmax(x, [2], [2])
+    assert np.isnan(out[0, :2]).all() and out[0, 2] == 1.0 and out[0, 3] == 0.0
+    ref = torch.softmax(torch.tensor(x).reshape(2, 2), -1).reshape(1, 4).numpy()
+    assert np.array_equal(np.isnan(out), np.isnan(ref))
+
+
+def test_softmax_with_gapped_prefix_sum():
+    src = np.arange(12, dtype=np.float32)[None]
+    out = oracle.blocked_softmax(src, [1, 1], [3, 4], accum=[0, 5, 12])     # gap of 2 after the first segment
+    np.testing.assert_allclose(out[0, 0:3], scipy.special.softmax(src[0, 0:3]), rtol=1e-6)
+    np.testing.assert_allclose(out[0, 5:9], scipy.special.softmax(src[0, 5:9]), rtol=1e-6)
+
+
+def test_softmax_backward_matches_autograd():
+    rng = np.random.default_rng(5)
+    rows, cols = [4, 7], [9, 3]
+    x = torch.tensor(rng.standard_normal((2, 57)), dtype=torch.float64, requires_grad=True)
+    dy = rng.standard_normal((2, 57)).astype(np.float32)
+    for scale in (1.0, 0.3):
+        y = torch.cat([torch.softmax(x[:, :36].reshape(2, 4, 9) * scale, -1).reshape(2, -1),
+                       torch.softmax(x[:, 36:].reshape(2, 7, 3) * scale, -1).reshape(2, -1)], -1)
+        (gx,) = torch.autograd.grad(y, x, torch.tensor(dy, dtype=torch.float64))
+        got = oracle.blocked_softmax_backward(y.detach().numpy().astype(np.float32), dy, rows, cols, scale)
+        np.testing.assert_allclose(got, gx.numpy(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("cfg", [1, 4])
+def test_c_oracle_and_per_segment_torch_agree(cfg):
+    w = workloads.make(cfg)
+    if cfg == 4:     # first 40 segments keep the C loops short
+        w.M, w.N, w.K = w.M[:40], w.N[:40], w.K[:40]
+    A, B = w.operands()
+    sc_t, pr_t = oracle.per_segment_torch(A, B, w.M, w.N, w.K, w.scale, want="both")
+    pr_c, sc_c = oracle.gemm_softmax(A.float().numpy(), B.float().numpy(), w.M, w.N, w.K, w.scale, return_scores=True)
+    np.testing.assert_allclose(sc_c, sc_t.numpy(), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(pr_c, pr_t.numpy(), rtol=1e-4, atol=1e-6)
+    ref = oracle.per_segment_torch_softmax(sc_t, w.M, w.N, w.scale)
+    np.testing.assert_allclose(ref.numpy(), pr_t.numpy(), rtol=1e-6, atol=1e-8)
