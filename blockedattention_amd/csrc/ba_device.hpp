@@ -96,15 +96,99 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) {
     return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
+// ------------------------------------------------------------ plan access
+// The plan is read-only while the compute kernels run, so it is read through
+// the constant address space: the loads become scalar loads (one per
+// wavefront, no vector registers, low latency).
+typedef const __attribute__((address_space(4))) int32_t *ConstI32;
+typedef const __attribute__((address_space(4))) int64_t *ConstI64;
+typedef const __attribute__((address_space(4))) SegRec *ConstSeg;
+typedef const __attribute__((address_space(4))) PlanHeader *ConstHdr;
+
+struct PlanRO {
+    ConstHdr hdr;
+    ConstSeg recs;
+    ConstI32 pfx[kNumPrefix];
+};
+
+__device__ __forceinline__ PlanRO plan_ro(const void *buf, int nseg) {
+    PlanRO v;
+    const size_t cap = (size_t)plan_cap(nseg);
+    uintptr_t p = (uintptr_t)buf;
+    v.hdr = (ConstHdr)p; p += sizeof(PlanHeader);
+    v.recs = (ConstSeg)p; p += cap * sizeof(SegRec);
+    for (int i = 0; i < kNumPrefix; ++i) { v.pfx[i] = (ConstI32)p; p += (cap + 4) * sizeof(int32_t); }
+    return v;
+}
+
+// One segment record, field by field (scalar loads when g is wave-uniform).
+__device__ __forceinline__ SegRec load_rec(ConstSeg recs, int g) {
+    const ConstI64 q = (ConstI64)(recs + g);
+    const ConstI32 w = (ConstI32)(recs + g);
+    SegRec r;
+    r.off1 = q[0]; r.off2 = q[1]; r.offO = q[2];
+    r.M = w[6]; r.N = w[7]; r.K = w[8]; r.packLen = w[9];
+    r.pad_[0] = r.pad_[1] = 0;
+    return r;
+}
+
 // Largest g in [0, n) with pfx[g] <= i, for an exclusive prefix array with
-// pfx[n] = total and 0 <= i < total.  Segments with no items are skipped.
-__device__ __forceinline__ int prefix_search(const int32_t *__restrict__ pfx, int n, int i) {
-    int lo = 0, hi = n;  // invariant: pfx[lo] <= i < pfx[hi]
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (pfx[mid] <= i) lo = mid; else hi = mid;
+// pfx[n] = total and 0 <= i < total (segments with no items are skipped).
+// 64-ary search: every lane tests one pivot per round, so 4096 segments take
+// two dependent loads instead of twelve.  The result is wave-uniform.
+template <typename PfxPtr> __device__ __forceinline__ int prefix_search(PfxPtr pfx, int n, int i) {
+    const int lane = lane_id();
+    int lo = 0, len = n;   // the answer lies in [lo, lo + len)
+    while (len > 1) {
+        const int step = (len + 63) >> 6;
+        const int idx = lo + (lane + 1) * step;
+        const bool le = idx < lo + len && pfx[idx] <= i;
+        const int cnt = __builtin_popcountll(__ballot(le));
+        const int end = lo + len;
+        lo += cnt * step;
+        len = min(step, end - lo);
     }
-    return lo;
+    return uniform(lo);
+}
+
+// ---------------------------------------------------------------- DPP scans
+// Inclusive prefix sum across the 64 lanes with data-parallel-primitive moves
+// (row shifts inside each 16-lane row, then two row broadcasts); no LDS traffic.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ int dpp_or_zero(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    v += dpp_or_zero<0x111, 0xf>(v);   // row_shr:1
+    v += dpp_or_zero<0x112, 0xf>(v);   // row_shr:2
+    v += dpp_or_zero<0x114, 0xf>(v);   // row_shr:4
+    v += dpp_or_zero<0x118, 0xf>(v);   // row_shr:8
+    v += dpp_or_zero<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ int64_t dpp64_or_zero(int64_t v) {
+    const uint32_t lo = (uint32_t)dpp_or_zero<CTRL, ROW_MASK>((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)dpp_or_zero<CTRL, ROW_MASK>((int)(uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ int64_t wave_inclusive_scan(int64_t v) {
+    v += dpp64_or_zero<0x111, 0xf>(v);
+    v += dpp64_or_zero<0x112, 0xf>(v);
+    v += dpp64_or_zero<0x114, 0xf>(v);
+    v += dpp64_or_zero<0x118, 0xf>(v);
+    v += dpp64_or_zero<0x142, 0xa>(v);
+    v += dpp64_or_zero<0x143, 0xc>(v);
+    return v;
+}
+// Maximum of non-negative ints over the wavefront (result in every lane).
+__device__ __forceinline__ int wave_max_nonneg(int v) {
+    v = max(v, dpp_or_zero<0x111, 0xf>(v));
+    v = max(v, dpp_or_zero<0x112, 0xf>(v));
+    v = max(v, dpp_or_zero<0x114, 0xf>(v));
+    v = max(v, dpp_or_zero<0x118, 0xf>(v));
+    v = max(v, dpp_or_zero<0x142, 0xa>(v));
+    v = max(v, dpp_or_zero<0x143, 0xc>(v));
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 }  // namespace ba

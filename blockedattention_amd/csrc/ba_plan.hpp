@@ -1,12 +1,13 @@
 // Plan: the device-resident result of the segment scheduler.  One contiguous
 // buffer; every compute kernel takes only this pointer plus the data pointers.
 //
-//   PlanHeader                                   (256 bytes)
-//   int64 off1[cap+1] off2[cap+1] offO[cap+1]    exclusive prefix sums (elements)
-//   int32 M[cap] N[cap] K[cap]                   segment shapes
-//   int32 prefix arrays, each [cap+1]            scanned work-item counts
+//   PlanHeader                    (256 bytes)
+//   SegRec recs[cap]              one 48-byte record per segment: offsets and shape
+//   int32 prefix arrays, each [cap+4]   scanned work-item counts, one array per kind
 //
-// cap = nseg rounded up so that every array starts 16-byte aligned.
+// cap = nseg rounded up so that every array starts 16-byte aligned.  The
+// compute kernels read the plan through scalar loads (it is never written
+// while they run, except the run_errors counter nobody reads back on the device).
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -56,20 +57,25 @@ static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 
 __host__ __device__ inline int64_t plan_cap(int64_t nseg) { return (nseg + 4) & ~int64_t(3); }
 
+// Everything a kernel needs to know about one segment, in one aligned record
+// (three 16-byte scalar loads).
+struct alignas(16) SegRec {
+    int64_t off1, off2, offO;   // element offsets of the segment in A, B and out (per head)
+    int32_t M, N, K;
+    int32_t packLen;            // > 0: first segment of a pack of this many segments
+    int32_t pad_[2];
+};
+static_assert(sizeof(SegRec) == 48, "SegRec must stay 48 bytes");
+
 struct PlanView {
     PlanHeader *hdr;
-    int64_t *off1, *off2, *offO;
-    int32_t *M, *N, *K;
+    SegRec *recs;
     int32_t *pfx[kNumPrefix];
-    // Segments that belong to a pack store the pack's segment count in packLen
-    // (leader) or 0 (follower / not packed).
-    int32_t *packLen;
 };
 
 __host__ __device__ inline size_t plan_bytes_for(int64_t nseg) {
     const size_t cap = (size_t)plan_cap(nseg);
-    return sizeof(PlanHeader) + 3 * (cap + 4) * sizeof(int64_t) + 4 * cap * sizeof(int32_t) +
-           kNumPrefix * (cap + 4) * sizeof(int32_t);
+    return sizeof(PlanHeader) + cap * sizeof(SegRec) + kNumPrefix * (cap + 4) * sizeof(int32_t);
 }
 
 __host__ __device__ inline PlanView plan_view(void *buf, int64_t nseg) {
@@ -77,13 +83,7 @@ __host__ __device__ inline PlanView plan_view(void *buf, int64_t nseg) {
     const size_t cap = (size_t)plan_cap(nseg);
     char *p = (char *)buf;
     v.hdr = (PlanHeader *)p; p += sizeof(PlanHeader);
-    v.off1 = (int64_t *)p; p += (cap + 4) * sizeof(int64_t);
-    v.off2 = (int64_t *)p; p += (cap + 4) * sizeof(int64_t);
-    v.offO = (int64_t *)p; p += (cap + 4) * sizeof(int64_t);
-    v.M = (int32_t *)p; p += cap * sizeof(int32_t);
-    v.N = (int32_t *)p; p += cap * sizeof(int32_t);
-    v.K = (int32_t *)p; p += cap * sizeof(int32_t);
-    v.packLen = (int32_t *)p; p += cap * sizeof(int32_t);
+    v.recs = (SegRec *)p; p += cap * sizeof(SegRec);
     for (int i = 0; i < kNumPrefix; ++i) { v.pfx[i] = (int32_t *)p; p += (cap + 4) * sizeof(int32_t); }
     return v;
 }

@@ -22,7 +22,7 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
         return;
     }
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
+    const PlanRO pv = plan_ro(a.plan, nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int lane = lane_id();
     const bool t1 = a.flags & kFlagTranspose1, t2 = a.flags & kFlagTranspose2;
@@ -38,15 +38,16 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
     for (int phase = 0; phase < 3; ++phase) {
         const int kind = kinds[phase];
         const int64_t per_head = hdr->totals[kind];
-        const int32_t *pfx = pv.pfx[kind];
+        const ConstI32 pfx = pv.pfx[kind];
         for (int64_t it = gw; it < per_head * a.H; it += nw) {
             const int64_t h = it / per_head;
             const int i = (int)(it - h * per_head);
             const int g0 = prefix_search(pfx, nseg, i);
-            const int members = kind == kPfxPack ? pv.packLen[g0] : 1;
+            const int members = kind == kPfxPack ? pv.recs[g0].packLen : 1;
             for (int j = 0; j < members; ++j) {
                 const int g = g0 + j;
-                const int M = pv.M[g], N = pv.N[g], K = pv.K[g];
+                const SegRec rec = load_rec(pv.recs, g);
+                const int M = rec.M, N = rec.N, K = rec.K;
                 int r0 = 0, c0 = 0, c1 = N;
                 if (kind == kPfxGemm) {
                     const int local = i - pfx[g];
@@ -56,9 +57,9 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
                 } else if (kind == kPfxSlow) {
                     r0 = (i - pfx[g]) * kStripRows;
                 }
-                const float *as = A + h * a.Dm1 + pv.off1[g];
-                const float *bs = B + h * a.Dm2 + pv.off2[g];
-                float *os = out + h * a.Dout + pv.offO[g];
+                const float *as = A + h * a.Dm1 + rec.off1;
+                const float *bs = B + h * a.Dm2 + rec.off2;
+                float *os = out + h * a.Dout + rec.offO;
                 const int rows = min(kStripRows, M - r0);
                 for (int col = c0 + lane; col < c1; col += 64) {
                     float acc[kStripRows];

@@ -291,12 +291,13 @@ __device__ __forceinline__ void wave_strip_dispatch(int nt, const Seg &s, const 
     else wave_strip<DT, 16, FUSED, F32OUT>(s, a, r0, c0, out_aligned);
 }
 
-__device__ __forceinline__ Seg load_seg(const PlanView &pv, int g, int64_t h, const RunArgs &a) {
+__device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
+    const SegRec r = load_rec(pv.recs, g);   // scalar loads
     Seg s;
-    s.M = uniform(pv.M[g]); s.N = uniform(pv.N[g]); s.K = uniform(pv.K[g]);
-    s.a = uniform64(h * a.Dm1 + pv.off1[g]);
-    s.b = uniform64(h * a.Dm2 + pv.off2[g]);
-    s.o = uniform64(h * a.Dout + pv.offO[g]);
+    s.M = r.M; s.N = r.N; s.K = r.K;
+    s.a = h * a.Dm1 + r.off1;
+    s.b = h * a.Dm2 + r.off2;
+    s.o = h * a.Dout + r.offO;
     return s;
 }
 
@@ -312,15 +313,15 @@ __device__ __forceinline__ void generic_seg_rows(const Seg &s, const RunArgs &a,
 // the tile's rows are the members' A rows back to back, its columns the
 // members' B rows back to back; only the block-diagonal products are kept.
 template <int DT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void wave_pack(const PlanView &pv, int g, int len, int64_t h, const RunArgs &a) {
+__device__ __forceinline__ void wave_pack(const PlanRO &pv, int g, int len, int64_t h, const RunArgs &a) {
     const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
-    const int K = pv.K[g];
+    const int K = pv.recs[g].K;
     int rowMem = -1, rowLoc = 0;                   // member and local row of tile row l16 (A side)
     int colMemL = -1, colLocL = 0;                 // member and local row of tile column l16 (B side)
     int cMem[4] = {-1, -1, -1, -1}, cLoc[4] = {0, 0, 0, 0};  // the same for the lane's four output columns
     int mAcc = 0, nAcc = 0;
     for (int j = 0; j < len; ++j) {
-        const int mj = pv.M[g + j], nj = pv.N[g + j];
+        const int mj = pv.recs[g + j].M, nj = pv.recs[g + j].N;
         if (rowMem < 0 && l16 < mAcc + mj) { rowMem = j; rowLoc = l16 - mAcc; }
         if (colMemL < 0 && l16 < nAcc + nj) { colMemL = j; colLocL = l16 - nAcc; }
 #pragma unroll
@@ -332,11 +333,11 @@ __device__ __forceinline__ void wave_pack(const PlanView &pv, int g, int len, in
     }
     // Rows / columns past the pack reuse the last member's last row (valid memory).
     const int am = rowMem >= 0 ? rowMem : len - 1;
-    const int al = rowMem >= 0 ? rowLoc : pv.M[g + len - 1] - 1;
+    const int al = rowMem >= 0 ? rowLoc : pv.recs[g + len - 1].M - 1;
     const int bm = colMemL >= 0 ? colMemL : len - 1;
-    const int bl = colMemL >= 0 ? colLocL : pv.N[g + len - 1] - 1;
-    const uint16_t *arow = (const uint16_t *)a.A + h * a.Dm1 + pv.off1[g + am] + (int64_t)al * K;
-    const uint16_t *brow = (const uint16_t *)a.B + h * a.Dm2 + pv.off2[g + bm] + (int64_t)bl * K;
+    const int bl = colMemL >= 0 ? colLocL : pv.recs[g + len - 1].N - 1;
+    const uint16_t *arow = (const uint16_t *)a.A + h * a.Dm1 + pv.recs[g + am].off1 + (int64_t)al * K;
+    const uint16_t *brow = (const uint16_t *)a.B + h * a.Dm2 + pv.recs[g + bm].off2 + (int64_t)bl * K;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < K; k0 += 32) {
         const int kk = k0 + q * 8;
@@ -372,8 +373,8 @@ __device__ __forceinline__ void wave_pack(const PlanView &pv, int g, int len, in
         for (int i = 0; i < 4; ++i) v[i] *= inv;
     }
     if (rowMem < 0) return;
-    const int Nr = pv.N[g + rowMem];
-    const int64_t e0 = h * a.Dout + pv.offO[g + rowMem] + (int64_t)rowLoc * Nr;
+    const int Nr = pv.recs[g + rowMem].N;
+    const int64_t e0 = h * a.Dout + pv.recs[g + rowMem].offO + (int64_t)rowLoc * Nr;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         if (keep[i]) store_one<DT>(a.out, e0 + cLoc[i], v[i], F32OUT);
@@ -428,22 +429,22 @@ __device__ __forceinline__ bool plan_matches(PlanHeader *hdr, const RunArgs &a) 
 // (transposed layouts, unaligned base pointers or head strides).
 template <int DT, bool FUSED>
 __device__ __attribute__((noinline)) void generic_phase(const RunArgs &a, bool everything, int64_t gw, int64_t nw) {
-    const PlanHeader *hdr = reinterpret_cast<const PlanHeader *>(a.plan);
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
+    const PlanRO pv = plan_ro(a.plan, nseg);
     const int kinds[5] = {kPfxSlow, kPfxPack, FUSED ? kPfxStrip : kPfxGemm, kPfxSplit, kPfxWide};
     const int nkinds = everything ? (FUSED ? 5 : 3) : 1;
     for (int ki = 0; ki < nkinds; ++ki) {
         const int kind = kinds[ki];
         const int64_t per_head = hdr->totals[kind];
-        const int32_t *pfx = pv.pfx[kind];
+        const ConstI32 pfx = pv.pfx[kind];
         for (int64_t it = gw; it < per_head * a.H; it += nw) {
             const int64_t h = it / per_head;
             const int i = (int)(it - h * per_head);
             const int g = prefix_search(pfx, nseg, i);
             const int local = i - pfx[g];
             if (kind == kPfxPack) {
-                const int len = pv.packLen[g];
+                const int len = pv.recs[g].packLen;
                 for (int j = 0; j < len; ++j) {
                     const Seg s = load_seg(pv, g + j, h, a);
                     generic_seg_rows<DT, FUSED>(s, a, 0, s.M, 0, s.N);
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(kItemThreads, 4) void wave_items_kernel(RunArgs a) 
     PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
     if (!plan_matches(hdr, a)) return;
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
+    const PlanRO pv = plan_ro(a.plan, nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int64_t gw = (int64_t)blockIdx.x * kItemWaves + wave;
     const int64_t nw = (int64_t)gridDim.x * kItemWaves;
@@ -476,18 +477,18 @@ __global__ __launch_bounds__(kItemThreads, 4) void wave_items_kernel(RunArgs a) 
     if (!mfma_ok) return;
     {
         const int64_t per_head = hdr->totals[kPfxPack];
-        const int32_t *pfx = pv.pfx[kPfxPack];
+        const ConstI32 pfx = pv.pfx[kPfxPack];
         for (int64_t it = gw; it < per_head * a.H; it += nw) {
             const int64_t h = it / per_head;
             const int i = (int)(it - h * per_head);
             const int g = prefix_search(pfx, nseg, i);
-            wave_pack<DT, FUSED, F32OUT>(pv, g, pv.packLen[g], h, a);
+            wave_pack<DT, FUSED, F32OUT>(pv, g, pv.recs[g].packLen, h, a);
         }
     }
     {
         const int kind = FUSED ? kPfxStrip : kPfxGemm;
         const int64_t per_head = hdr->totals[kind];
-        const int32_t *pfx = pv.pfx[kind];
+        const ConstI32 pfx = pv.pfx[kind];
         for (int64_t it = gw; it < per_head * a.H; it += nw) {
             const int64_t h = it / per_head;
             const int i = (int)(it - h * per_head);
@@ -517,11 +518,11 @@ __global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
     PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
     if (!(a.flags & kFlagMfmaOk) || !plan_matches(hdr, a)) return;
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
+    const PlanRO pv = plan_ro(a.plan, nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const bool out_aligned = ((uintptr_t)a.out & 15) == 0;
     const int64_t per_head = hdr->totals[kPfxSplit];
-    const int32_t *pfx = pv.pfx[kPfxSplit];
+    const ConstI32 pfx = pv.pfx[kPfxSplit];
     float c = a.scale * kLog2e;
     const bool neg = c < 0.f;
     if (neg) c = -c;
@@ -570,11 +571,11 @@ __global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
     PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
     if (!(a.flags & kFlagMfmaOk) || !plan_matches(hdr, a)) return;
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
+    const PlanRO pv = plan_ro(a.plan, nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const bool out_aligned = ((uintptr_t)a.out & 15) == 0;
     const int64_t per_head = hdr->totals[kPfxWide];
-    const int32_t *pfx = pv.pfx[kPfxWide];
+    const ConstI32 pfx = pv.pfx[kPfxWide];
     float c = a.scale * kLog2e;
     const bool neg = c < 0.f;
     if (neg) c = -c;

@@ -9,6 +9,13 @@
 
 namespace ba {
 
+__device__ __forceinline__ int32_t readlane_t(int32_t v, int l) { return __builtin_amdgcn_readlane(v, l); }
+__device__ __forceinline__ int64_t readlane_t(int64_t v, int l) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, l);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)v >> 32), l);
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 constexpr int kSchedThreads = 1024;
 constexpr int kSchedWaves = kSchedThreads / 64;
 
@@ -21,42 +28,29 @@ struct SchedArgs {
     int64_t *a1, *a2, *aO;
 };
 
-// Inclusive scan inside one wavefront.
-template <typename T> __device__ __forceinline__ T wave_inclusive_scan(T v) {
-    const int lane = lane_id();
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        T u = __shfl_up(v, o);
-        if (lane >= o) v += u;
-    }
-    return v;
-}
-
-// Exclusive scan of NQ quantities over the workgroup; total[] receives the sums.
-// lds must hold kSchedWaves * NQ entries.  Ends with a barrier-free state in
-// which lds may be reused after the next __syncthreads().
+// Exclusive scan of NQ quantities over the workgroup.  Wavefront-level DPP
+// scans, then the 16 wavefront totals are scanned by lanes 0..15 of every
+// wavefront (one row of DPP shifts).  lds holds NQ * kSchedWaves entries and
+// is free for reuse after the next __syncthreads().  One barrier.
 template <typename T, int NQ>
 __device__ __forceinline__ void block_exclusive_scan(T (&v)[NQ], T (&total)[NQ], T *lds) {
-    const int wave = threadIdx.x >> 6, lane = lane_id();
+    const int wave = uniform((int)(threadIdx.x >> 6)), lane = lane_id();
     T incl[NQ];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
         incl[q] = wave_inclusive_scan(v[q]);
-        if (lane == 63) lds[wave * NQ + q] = incl[q];
+        if (lane == 63) lds[q * kSchedWaves + wave] = incl[q];
     }
     __syncthreads();
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-        T base = 0, tot = 0;
-        for (int w = 0; w < kSchedWaves; ++w) {
-            const T s = lds[w * NQ + q];
-            if (w < wave) base += s;
-            tot += s;
-        }
-        v[q] = base + incl[q] - v[q];
-        total[q] = tot;
+        T t = lane < kSchedWaves ? lds[q * kSchedWaves + lane] : T(0);
+        t = wave_inclusive_scan(t);                    // lanes 0..15 now hold the scan over wavefronts
+        const T upto = readlane_t(t, kSchedWaves - 1);
+        const T before = wave == 0 ? T(0) : readlane_t(t, wave - 1);
+        v[q] = before + incl[q] - v[q];
+        total[q] = upto;
     }
-    __syncthreads();
 }
 
 __device__ __forceinline__ int64_t isqrt64(int64_t v) {
@@ -92,18 +86,18 @@ __device__ __forceinline__ bool derive_lists(int64_t mk, int64_t nk, int64_t mn,
 __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     __shared__ int64_t sScan64[kSchedWaves * 3];
     __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
-    __shared__ int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads], sPack[kSchedThreads];
-    __shared__ int32_t sMax[3], sBad;
+    __shared__ __attribute__((aligned(16))) int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads];
+    __shared__ int32_t sPack[kSchedThreads];
+    __shared__ int32_t sRed[kSchedWaves][4];
 
     const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6), lane = lane_id();
     const int64_t nseg = a.nseg;
     PlanView pv = plan_view(a.plan, nseg);
-    if (tid == 0) { sMax[0] = sMax[1] = sMax[2] = 0; sBad = 0; }
-    __syncthreads();
 
     int64_t base64[3] = {0, 0, 0};
     int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0};
-    int64_t rows_total = 0;
+    int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
 
     for (int64_t chunk = 0; chunk < nseg || chunk == 0; chunk += kSchedThreads) {
@@ -129,8 +123,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             }
             const int64_t lim = int64_t(1) << 30;
             bad = bad || m < 0 || n < 0 || k < 0 || m >= lim || n >= lim || k >= lim;
-            if (bad) { m = n = k = 0; atomicAdd(&sBad, 1); }
+            if (bad) { m = n = k = 0; }
         }
+        const int32_t mi = (int32_t)m, ni = (int32_t)n, ki = (int32_t)k;
         // Offsets first: alignment decides which path a segment takes.
         int64_t v64[3] = {m * k, n * k, m * n}, t64[3] = {0, 0, 0};
         if (!offsets_given) {
@@ -141,45 +136,55 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         // offsets of the buffer instructions.
         const int64_t lim31 = int64_t(1) << 31;
         const bool aligned = ((k | o1 | o2) & 7) == 0 && m * k < lim31 && n * k < lim31 && m * n < lim31 / 2;
-        sM[tid] = (int32_t)m; sN[tid] = (int32_t)n; sK[tid] = aligned ? (int32_t)k : -1; sPack[tid] = 0;
-        __syncthreads();
 
         // Packs: inside each aligned window of 16 segments, greedily join
         // consecutive tiny aligned segments (same K, sum M <= 16, sum N <= 16).
-        if (a.kind == 0 && (tid & 15) == 0) {
-            int i = 0;
-            while (i < 16) {
-                const int s = tid + i;
-                int len = 0, sumM = 0, sumN = 0;
-                const int k0 = sK[s];
-                while (i + len < 16) {
-                    const int mm = sM[s + len], nn = sN[s + len];
-                    if (mm < 1 || nn < 1 || sK[s + len] != k0 || k0 < 1) break;
-                    if (sumM + mm > kPackDim || sumN + nn > kPackDim) break;
-                    sumM += mm; sumN += nn; ++len;
+        // The first lane of every window walks its 16 entries in registers.
+        int32_t pack = 0;
+        if (a.kind == 0) {
+            sM[tid] = mi; sN[tid] = ni; sK[tid] = aligned ? ki : -1; sPack[tid] = 0;
+            __syncthreads();
+            if ((tid & 15) == 0) {
+                int32_t wm[16], wn[16], wk[16];
+#pragma unroll
+                for (int j = 0; j < 16; j += 4) {
+                    const int4 vm = *reinterpret_cast<const int4 *>(&sM[tid + j]);
+                    const int4 vn = *reinterpret_cast<const int4 *>(&sN[tid + j]);
+                    const int4 vk = *reinterpret_cast<const int4 *>(&sK[tid + j]);
+                    wm[j] = vm.x; wm[j + 1] = vm.y; wm[j + 2] = vm.z; wm[j + 3] = vm.w;
+                    wn[j] = vn.x; wn[j + 1] = vn.y; wn[j + 2] = vn.z; wn[j + 3] = vn.w;
+                    wk[j] = vk.x; wk[j + 1] = vk.y; wk[j + 2] = vk.z; wk[j + 3] = vk.w;
                 }
-                if (len >= 2) {
-                    sPack[s] = len;
-                    for (int j = 1; j < len; ++j) sPack[s + j] = -1;
-                    i += len;
-                } else {
-                    i += 1;
+                int start = 0, len = 0, sumM = 0, sumN = 0, kcur = 0;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const bool ok = wm[j] >= 1 && wn[j] >= 1 && wk[j] >= 1;
+                    const bool fits = ok && len > 0 && wk[j] == kcur && sumM + wm[j] <= kPackDim &&
+                                      sumN + wn[j] <= kPackDim;
+                    if (fits) {
+                        sumM += wm[j]; sumN += wn[j]; ++len;
+                        sPack[tid + j] = -1;
+                    } else {
+                        if (len >= 2) sPack[tid + start] = len;
+                        start = j; len = ok ? 1 : 0; sumM = wm[j]; sumN = wn[j]; kcur = wk[j];
+                    }
                 }
+                if (len >= 2) sPack[tid + start] = len;
             }
+            __syncthreads();
+            pack = sPack[tid];
         }
-        __syncthreads();
 
-        const int32_t pack = sPack[tid];
-        const int32_t strips = (n >= 1) ? (int32_t)((m + kStripRows - 1) / kStripRows) : 0;
-        const int64_t chunks = (n + kWaveCols - 1) / kWaveCols;
+        const int32_t strips = (ni >= 1) ? (mi + kStripRows - 1) / kStripRows : 0;
+        const int32_t chunks = (ni + kWaveCols - 1) / kWaveCols;
         const bool packed = pack != 0;
         const bool mfma_ok = aligned && !packed;
         int32_t v32[kNumPrefix], t32[kNumPrefix];
-        v32[kPfxGemm] = mfma_ok ? (int32_t)(strips * chunks) : 0;
-        v32[kPfxStrip] = (mfma_ok && n <= kWaveCols) ? strips : 0;
-        v32[kPfxSplit] = (mfma_ok && n > kWaveCols && n <= kSplitCols) ? strips : 0;
-        v32[kPfxWide] = (mfma_ok && n > kSplitCols) ? strips : 0;
-        v32[kPfxRows] = n >= 1 ? (int32_t)m : 0;
+        v32[kPfxGemm] = mfma_ok ? strips * chunks : 0;
+        v32[kPfxStrip] = (mfma_ok && ni <= kWaveCols) ? strips : 0;
+        v32[kPfxSplit] = (mfma_ok && ni > kWaveCols && ni <= kSplitCols) ? strips : 0;
+        v32[kPfxWide] = (mfma_ok && ni > kSplitCols) ? strips : 0;
+        v32[kPfxRows] = ni >= 1 ? mi : 0;
         v32[kPfxPack] = pack > 0 ? 1 : 0;
         v32[kPfxSlow] = aligned ? 0 : strips;
         if (a.kind == 1) {
@@ -190,9 +195,11 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         block_exclusive_scan<int32_t, kNumPrefix>(v32, t32, sScan32);
 
         if (live) {
-            pv.off1[g] = o1; pv.off2[g] = o2; pv.offO[g] = oO;
-            pv.M[g] = (int32_t)m; pv.N[g] = (int32_t)n; pv.K[g] = (int32_t)k;
-            pv.packLen[g] = pack > 0 ? pack : 0;
+            SegRec rec;
+            rec.off1 = o1; rec.off2 = o2; rec.offO = oO;
+            rec.M = mi; rec.N = ni; rec.K = ki; rec.packLen = pack > 0 ? pack : 0;
+            rec.pad_[0] = rec.pad_[1] = 0;
+            pv.recs[g] = rec;
 #pragma unroll
             for (int q = 0; q < kNumPrefix; ++q) pv.pfx[q][g] = base32[q] + v32[q];
             if (!offsets_given) {
@@ -205,9 +212,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
                 if (a.N) a.N[g] = bad ? -1 : n;
                 if (a.K) a.K[g] = bad ? -1 : k;
             }
-            atomicMax(&sMax[0], (int32_t)m); atomicMax(&sMax[1], (int32_t)n); atomicMax(&sMax[2], (int32_t)k);
         }
-        rows_total += t32[kPfxRows];
+        maxM = max(maxM, mi); maxN = max(maxN, ni); maxK = max(maxK, ki); nbad += bad ? 1 : 0;
 #pragma unroll
         for (int q = 0; q < kNumPrefix; ++q) base32[q] += t32[q];
         if (!offsets_given) {
@@ -215,7 +221,14 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             for (int q = 0; q < 3; ++q) base64[q] += t64[q];
         }
         if (nseg == 0) break;
+        __syncthreads();   // the scan scratch is rewritten by the next pass
     }
+
+    // Shape maxima and the count of rejected segments: DPP reduction per
+    // wavefront, then thread 0 folds the 16 partial results.
+    maxM = wave_max_nonneg(maxM); maxN = wave_max_nonneg(maxN); maxK = wave_max_nonneg(maxK);
+    nbad = __builtin_amdgcn_readlane(wave_inclusive_scan(nbad), 63);
+    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; }
     __syncthreads();
 
     if (tid == 0) {
@@ -230,7 +243,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             if (a.a2) a.a2[nseg] = D2;
             if (a.aO) a.aO[nseg] = DO;
         }
-        pv.off1[nseg] = D1; pv.off2[nseg] = D2; pv.offO[nseg] = DO;
+        int32_t rM = 0, rN = 0, rK = 0, rBad = 0;
+        for (int w = 0; w < kSchedWaves; ++w) {
+            rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3];
+        }
         for (int q = 0; q < kNumPrefix; ++q) pv.pfx[q][nseg] = base32[q];
         PlanHeader *h = pv.hdr;
         h->magic = kPlanMagic;
@@ -238,10 +254,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->cap = (int32_t)plan_cap(nseg);
         h->kind = a.kind;
         h->Dm1 = D1; h->Dm2 = D2; h->Dout = DO;
-        h->total_rows = rows_total;
+        h->total_rows = base32[kPfxRows];
         for (int q = 0; q < 8; ++q) h->totals[q] = q < kNumPrefix ? base32[q] : 0;
-        h->max_M = sMax[0]; h->max_N = sMax[1]; h->max_K = sMax[2];
-        h->bad_segments = sBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
+        h->max_M = rM; h->max_N = rN; h->max_K = rK;
+        h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
         h->run_errors = 0;
     }
 }

@@ -52,8 +52,8 @@ template <int DT> __global__ __launch_bounds__(kSoftmaxThreads) void softmax_row
         return;
     }
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
-    const int32_t *pfx = pv.pfx[kPfxRows];
+    const PlanRO pv = plan_ro(a.plan, nseg);
+    const ConstI32 pfx = pv.pfx[kPfxRows];
     const int64_t per_head = hdr->totals[kPfxRows];
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int lane = lane_id();
@@ -69,8 +69,9 @@ template <int DT> __global__ __launch_bounds__(kSoftmaxThreads) void softmax_row
         const int i = (int)(it - h * per_head);
         const int g = prefix_search(pfx, nseg, i);
         const int r = i - pfx[g];
-        const int cols = pv.N[g];
-        const int64_t e0 = h * a.Dsrc + pv.offO[g] + (int64_t)r * cols;
+        const SegRec rec = load_rec(pv.recs, g);
+        const int cols = rec.N;
+        const int64_t e0 = h * a.Dsrc + rec.offO + (int64_t)r * cols;
         const T *x = src + e0;
         T *y = dst + e0;
         if (cols <= 64 * kRegs) {
@@ -156,8 +157,8 @@ template <int DT> __global__ __launch_bounds__(kSoftmaxThreads) void softmax_row
         return;
     }
     const int nseg = hdr->nseg;
-    const PlanView pv = plan_view(a.plan, nseg);
-    const int32_t *pfx = pv.pfx[kPfxRows];
+    const PlanRO pv = plan_ro(a.plan, nseg);
+    const ConstI32 pfx = pv.pfx[kPfxRows];
     const int64_t per_head = hdr->totals[kPfxRows];
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int lane = lane_id();
@@ -169,8 +170,9 @@ template <int DT> __global__ __launch_bounds__(kSoftmaxThreads) void softmax_row
         const int i = (int)(it - h * per_head);
         const int g = prefix_search(pfx, nseg, i);
         const int r = i - pfx[g];
-        const int cols = pv.N[g];
-        const int64_t e0 = h * a.Dsrc + pv.offO[g] + (int64_t)r * cols;
+        const SegRec rec = load_rec(pv.recs, g);
+        const int cols = rec.N;
+        const int64_t e0 = h * a.Dsrc + rec.offO + (int64_t)r * cols;
         const T *y = ys + e0, *dy = dys + e0;
         T *dx = dxs + e0;
         if (cols <= 64 * kRegs) {
