@@ -47,11 +47,12 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = os.environ.get("BLOCKEDATTN_LIB", LIB_PATH)   # lets a caller point at another build of the library
+    if not os.path.exists(path):
         raise BlockedAttentionError(
-            f"{LIB_PATH} is missing: build it with `python -m blockedattention_amd.build lib` "
+            f"{path} is missing: build it with `python -m blockedattention_amd.build lib` "
             "(there is no CPU or PyTorch fallback)")
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
     lib.ba_status_string.restype = ctypes.c_char_p
     lib.ba_status_string.argtypes = [i32]
@@ -65,13 +66,13 @@ def load():
     lib.ba_plan_read.restype = i32
     lib.ba_plan_read.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
     lib.ba_varlen_gemm.restype = i32
-    lib.ba_varlen_gemm.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
+    lib.ba_varlen_gemm.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
     lib.ba_blocked_softmax.restype = i32
-    lib.ba_blocked_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, i64, i64, f32, vp]
+    lib.ba_blocked_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, i64, i64, f32, vp]
     lib.ba_blocked_softmax_backward.restype = i32
-    lib.ba_blocked_softmax_backward.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i64, i64, f32, vp]
+    lib.ba_blocked_softmax_backward.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i64, i64, f32, vp]
     lib.ba_gemm_softmax.restype = i32
-    lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
+    lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
     _lib = lib
     return lib
 
@@ -158,28 +159,28 @@ def plan_softmax(nseg, device, rowList, colList, accum=None, accum_given=False):
 
 
 def varlen_gemm(plan, A, B, out, H, Dm1, Dm2, Dout, transpose1=False, transpose2=False):
-    st = load().ba_varlen_gemm(plan.ptr, plan._hint(), dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out), H, Dm1, Dm2,
+    st = load().ba_varlen_gemm(plan.ptr, plan._hint(), plan.nseg, dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out), H, Dm1, Dm2,
                                Dout, int(transpose1), int(transpose2), _stream())
     check(st, "ba_varlen_gemm")
     return out
 
 
 def blocked_softmax(plan, src, dst, H, Dsrc, scale=1.0):
-    st = load().ba_blocked_softmax(plan.ptr, plan._hint(), dtype_code(src.dtype), _ptr(src), _ptr(dst), H, Dsrc,
+    st = load().ba_blocked_softmax(plan.ptr, plan._hint(), plan.nseg, dtype_code(src.dtype), _ptr(src), _ptr(dst), H, Dsrc,
                                    float(scale), _stream())
     check(st, "ba_blocked_softmax")
     return dst
 
 
 def blocked_softmax_backward(plan, y, dy, dx, H, Dsrc, scale=1.0):
-    st = load().ba_blocked_softmax_backward(plan.ptr, plan._hint(), dtype_code(y.dtype), _ptr(y), _ptr(dy), _ptr(dx),
+    st = load().ba_blocked_softmax_backward(plan.ptr, plan._hint(), plan.nseg, dtype_code(y.dtype), _ptr(y), _ptr(dy), _ptr(dx),
                                             H, Dsrc, float(scale), _stream())
     check(st, "ba_blocked_softmax_backward")
     return dx
 
 
 def gemm_softmax(plan, A, B, out, H, Dm1, Dm2, Dout, scale=1.0):
-    st = load().ba_gemm_softmax(plan.ptr, plan._hint(), dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out),
+    st = load().ba_gemm_softmax(plan.ptr, plan._hint(), plan.nseg, dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out),
                                 dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
     check(st, "ba_gemm_softmax")
     return out

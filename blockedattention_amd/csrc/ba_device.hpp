@@ -127,8 +127,8 @@ __device__ __forceinline__ SegRec load_rec(ConstSeg recs, int g) {
     const ConstI32 w = (ConstI32)(recs + g);
     SegRec r;
     r.off1 = q[0]; r.off2 = q[1]; r.offO = q[2];
-    r.M = w[6]; r.N = w[7]; r.K = w[8]; r.packLen = w[9];
-    r.pad_[0] = r.pad_[1] = 0;
+    r.M = w[6]; r.N = w[7]; r.K = w[8]; r.packLen = w[9]; r.kind = w[10];
+    r.pad_ = 0;
     return r;
 }
 

@@ -23,6 +23,7 @@ struct RunArgs {
     int64_t H, Dm1, Dm2, Dout;
     float scale;
     int flags;
+    int lds_blocks;   // 1 KiB operand blocks of dynamic LDS given to the segment kernel
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,
@@ -30,13 +31,14 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
 
 // mode 0 = GEMM only, 1 = fused GEMM + softmax.  dtype BA_F16 / BA_BF16.
 // info: optional host copy of the plan summary (from ba_plan_read), or nullptr.
-int launch_strips(int dtype, int fused, const RunArgs &args, const ba_plan_info *info, hipStream_t stream);
-int launch_gemm_f32(const RunArgs &args, const ba_plan_info *info, hipStream_t stream);
-int launch_softmax(int dtype, void *plan, const void *src, void *dst, int64_t H, int64_t Dsrc, float scale,
-                   const ba_plan_info *info, hipStream_t stream);
+int launch_strips(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
+                  hipStream_t stream);
+int launch_gemm_f32(const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
+int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,
+                   float scale, const ba_plan_info *info, hipStream_t stream);
 
-int launch_softmax_backward(int dtype, void *plan, const void *y, const void *dy, void *dx, int64_t H, int64_t Dsrc,
-                            float scale, const ba_plan_info *info, hipStream_t stream);
+int launch_softmax_backward(int dtype, void *plan, int64_t nseg, const void *y, const void *dy, void *dx, int64_t H,
+                            int64_t Dsrc, float scale, const ba_plan_info *info, hipStream_t stream);
 
 // Number of compute units of the current device (cached per device).
 int device_cu_count();

@@ -24,7 +24,7 @@ constexpr int kPackDim = 16;      // a pack of tiny segments fits one 16x16 MFMA
 // Kinds of scanned work-item counts.  Every kind except kPfxRows and kPfxSlow
 // counts aligned segments only (see below).
 enum PrefixKind {
-    kPfxGemm = 0,   // GEMM only: ceil(M/16) * ceil(N/256) per segment
+    kPfxGemm = 0,   // GEMM only, N > 256: ceil(M/16) * ceil(N/256) per segment
     kPfxStrip = 1,  // fused, N <= 256 and not packed: ceil(M/16)
     kPfxSplit = 2,  // fused, 256 < N <= 4096: ceil(M/16)
     kPfxWide = 3,   // fused, N > 4096: ceil(M/16)
@@ -57,13 +57,25 @@ static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 
 __host__ __device__ inline int64_t plan_cap(int64_t nseg) { return (nseg + 4) & ~int64_t(3); }
 
+// How a segment is processed.
+enum SegKind : int32_t {
+    kSegEmpty = 0,       // no rows or no columns: no work
+    kSegStrip = 1,       // aligned, N <= 256: one wavefront per 16-row strip, scores in registers
+    kSegPackLead = 2,    // first segment of a pack of tiny segments sharing one MFMA tile
+    kSegPackFollow = 3,  // later member of a pack (processed with its leader)
+    kSegSplit = 4,       // aligned, 256 < N <= 4096
+    kSegWide = 5,        // aligned, N > 4096
+    kSegSlow = 6         // not 16-byte aligned (K % 8, odd offsets) or too large for 32-bit offsets
+};
+
 // Everything a kernel needs to know about one segment, in one aligned record
 // (three 16-byte scalar loads).
 struct alignas(16) SegRec {
     int64_t off1, off2, offO;   // element offsets of the segment in A, B and out (per head)
     int32_t M, N, K;
     int32_t packLen;            // > 0: first segment of a pack of this many segments
-    int32_t pad_[2];
+    int32_t kind;               // SegKind
+    int32_t pad_;
 };
 static_assert(sizeof(SegRec) == 48, "SegRec must stay 48 bytes");
 

@@ -96,53 +96,57 @@ __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_pla
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 
-__attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_plan_info *info, int dtype,
+__attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_plan_info *info, int64_t nseg,
+                                                          int dtype,
                                                           const void *A, const void *B, void *out, int64_t H,
                                                           int64_t Dm1, int64_t Dm2, int64_t Dout, int transpose1,
                                                           int transpose2, ba_stream_t stream) {
-    if (!plan || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
-    if (H == 0 || Dout == 0) return BA_OK;
+    if (!plan || nseg < 0 || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
     if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0};
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0, 0};
     if (transpose1) args.flags |= kFlagTranspose1;
     if (transpose2) args.flags |= kFlagTranspose2;
     args.flags |= mfma_flag(args);
-    if (dtype == BA_F32) return launch_gemm_f32(args, info, (hipStream_t)stream);
-    return launch_strips(dtype, 0, args, info, (hipStream_t)stream);
+    if (dtype == BA_F32) return launch_gemm_f32(args, nseg, info, (hipStream_t)stream);
+    return launch_strips(dtype, 0, args, nseg, info, (hipStream_t)stream);
 }
 
-__attribute__((visibility("default"))) int ba_blocked_softmax(void *plan, const ba_plan_info *info, int dtype,
+__attribute__((visibility("default"))) int ba_blocked_softmax(void *plan, const ba_plan_info *info, int64_t nseg,
+                                                              int dtype,
                                                               const void *src, void *dst, int64_t H, int64_t Dsrc,
                                                               float scale, ba_stream_t stream) {
-    if (!plan || H < 0 || Dsrc < 0) return BA_ERR_INVALID_ARG;
-    if (H == 0 || Dsrc == 0) return BA_OK;
+    if (!plan || nseg < 0 || H < 0 || Dsrc < 0) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dsrc == 0 || nseg == 0) return BA_OK;
     if (!src || !dst) return BA_ERR_INVALID_ARG;
-    return launch_softmax(dtype, plan, src, dst, H, Dsrc, scale, info, (hipStream_t)stream);
+    return launch_softmax(dtype, plan, nseg, src, dst, H, Dsrc, scale, info, (hipStream_t)stream);
 }
 
 __attribute__((visibility("default"))) int ba_blocked_softmax_backward(void *plan, const ba_plan_info *info,
-                                                                       int dtype, const void *y, const void *dy,
+                                                                       int64_t nseg, int dtype, const void *y,
+                                                                       const void *dy,
                                                                        void *dx, int64_t H, int64_t Dsrc,
                                                                        float scale, ba_stream_t stream) {
-    if (!plan || H < 0 || Dsrc < 0) return BA_ERR_INVALID_ARG;
-    if (H == 0 || Dsrc == 0) return BA_OK;
+    if (!plan || nseg < 0 || H < 0 || Dsrc < 0) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dsrc == 0 || nseg == 0) return BA_OK;
     if (!y || !dy || !dx) return BA_ERR_INVALID_ARG;
-    return launch_softmax_backward(dtype, plan, y, dy, dx, H, Dsrc, scale, info, (hipStream_t)stream);
+    return launch_softmax_backward(dtype, plan, nseg, y, dy, dx, H, Dsrc, scale, info, (hipStream_t)stream);
 }
 
-__attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_plan_info *info, int dtype,
+__attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_plan_info *info, int64_t nseg,
+                                                           int dtype,
                                                            const void *A, const void *B, void *out, int out_dtype,
                                                            int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
                                                            float scale, ba_stream_t stream) {
-    if (!plan || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (!plan || nseg < 0 || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
     if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
     if (out_dtype != dtype && out_dtype != BA_F32) return BA_ERR_UNSUPPORTED;
-    if (H == 0 || Dout == 0) return BA_OK;
+    if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
     if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0};
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0};
     args.flags |= mfma_flag(args);
     if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
-    return launch_strips(dtype, 1, args, info, (hipStream_t)stream);
+    return launch_strips(dtype, 1, args, nseg, info, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -34,24 +34,21 @@ struct Seg {
     int64_t a, b, o;  // element offsets of the segment inside A, B, out (head included)
 };
 
-// Buffer resources of one segment.  Every operand load and result store goes
-// through a raw buffer descriptor whose range is exactly the segment: the
-// address is one 32-bit lane offset plus a scalar offset, and anything past the
-// segment's end (rows >= M of a ragged strip, columns >= N of a ragged tile)
-// reads as zero or is dropped by the hardware instead of being clamped in code.
+// Buffer resources of one segment.  Operand loads go through a raw buffer
+// descriptor whose range is exactly the segment: the address is one 32-bit lane
+// offset plus a scalar offset, and anything past the segment's end (rows >= M
+// of a ragged strip, columns >= N of a ragged tile) reads as zero instead of
+// being clamped in code.
 struct SegRes {
-    __amdgpu_buffer_rsrc_t a, b, o;
+    __amdgpu_buffer_rsrc_t a, b;
 };
 
 constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
 
-template <int OUT_BYTES>
-__device__ __forceinline__ SegRes make_res(const Seg &s, const void *A, const void *B, void *out) {
+__device__ __forceinline__ SegRes make_res(const Seg &s, const void *A, const void *B) {
     SegRes r;
     r.a = __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)A + s.a), 0, s.M * s.K * 2, kRsrcFlags);
     r.b = __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)B + s.b), 0, s.N * s.K * 2, kRsrcFlags);
-    r.o = __builtin_amdgcn_make_buffer_rsrc((void *)((char *)out + s.o * OUT_BYTES), 0, s.M * s.N * OUT_BYTES,
-                                            kRsrcFlags);
     return r;
 }
 
@@ -215,45 +212,46 @@ __device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int N, in
 
 // ------------------------------------------------------------------- stores
 // Writes acc[t][i] * factor for rows < M and columns < N.  The lane's four
-// columns are consecutive in memory: one 8-byte (16-bit output) or 16-byte
-// (fp32 output) store when the address allows it, element stores otherwise.
+// columns are consecutive in memory and go out as ONE 8-byte (16-bit output)
+// or 16-byte (fp32 output) store whatever the address: row starts are only
+// element-aligned (odd N), and the memory pipeline takes vector stores at any
+// element alignment.  Only the ragged last tile of a row falls back to
+// element stores.
+typedef u32x2 __attribute__((aligned(2))) u32x2_unaligned;
+typedef f32x4 __attribute__((aligned(4))) f32x4_unaligned;
+
 template <int DT, int NT, bool F32OUT>
-__device__ __forceinline__ void store_rows(const f32x4 (&acc)[kMaxTiles], const Seg &s, const SegRes &res, int r0,
-                                           int c0, float factor, bool out_aligned) {
+__device__ __forceinline__ void store_rows(const f32x4 (&acc)[kMaxTiles], const Seg &s, void *__restrict__ out, int r0,
+                                           int c0, float factor) {
     const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
     const int r = r0 + l16;
     if (r >= s.M) return;
-    const int e0 = r * s.N;                 // element offset of the row inside the segment
-    const int phase = (int)(s.o & 3);       // alignment of the segment start in elements
+    const int64_t e0 = s.o + (int64_t)r * s.N;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int col = c0 + t * 16 + q * 4;
         if (col >= s.N) continue;
-        const int e = e0 + col;
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = acc[t][i] * factor;
-        const bool vec = col + 3 < s.N && ((e + phase) & 3) == 0 && out_aligned;
         if (F32OUT) {
-            if (vec) {
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, f32x4{v[0], v[1], v[2], v[3]}),
-                                                       res.o, e * 4, 0, 0);
+            float *o = reinterpret_cast<float *>(out) + e0 + col;
+            if (col + 3 < s.N) {
+                *reinterpret_cast<f32x4_unaligned *>(o) = f32x4{v[0], v[1], v[2], v[3]};
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (col + i < s.N)
-                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[i]), res.o, (e + i) * 4,
-                                                              0, 0);
+                    if (col + i < s.N) o[i] = v[i];
             }
         } else {
-            if (vec) {
-                __builtin_amdgcn_raw_buffer_store_b64(
-                    u32x2{Elem<DT>::pack2(v[0], v[1]), Elem<DT>::pack2(v[2], v[3])}, res.o, e * 2, 0, 0);
+            uint16_t *o = reinterpret_cast<uint16_t *>(out) + e0 + col;
+            if (col + 3 < s.N) {
+                *reinterpret_cast<u32x2_unaligned *>(o) =
+                    u32x2{Elem<DT>::pack2(v[0], v[1]), Elem<DT>::pack2(v[2], v[3])};
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (col + i < s.N)
-                        __builtin_amdgcn_raw_buffer_store_b16(Elem<DT>::from_float(v[i]), res.o, (e + i) * 2, 0, 0);
+                    if (col + i < s.N) o[i] = Elem<DT>::from_float(v[i]);
             }
         }
     }
@@ -266,9 +264,9 @@ template <int NT> __device__ __forceinline__ void negate(f32x4 (&acc)[kMaxTiles]
 
 // One wavefront, one strip, everything in registers.
 template <int DT, int NT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void wave_strip(const Seg &s, const RunArgs &a, int r0, int c0, bool out_aligned) {
+__device__ __forceinline__ void wave_strip(const Seg &s, const RunArgs &a, int r0, int c0) {
     f32x4 acc[kMaxTiles];
-    const SegRes res = make_res<F32OUT ? 4 : 2>(s, a.A, a.B, a.out);
+    const SegRes res = make_res(s, a.A, a.B);
     stage_scores<DT, NT>(acc, s, res, r0, c0);
     float factor = 1.f;
     if (FUSED) {
@@ -278,17 +276,16 @@ __device__ __forceinline__ void wave_strip(const Seg &s, const RunArgs &a, int r
         local_softmax<NT>(acc, s.N, c0, c, m, l);
         factor = 1.f / l;
     }
-    store_rows<DT, NT, F32OUT>(acc, s, res, r0, c0, factor, out_aligned);
+    store_rows<DT, NT, F32OUT>(acc, s, a.out, r0, c0, factor);
 }
 
 template <int DT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void wave_strip_dispatch(int nt, const Seg &s, const RunArgs &a, int r0, int c0,
-                                                    bool out_aligned) {
-    if (nt <= 1) wave_strip<DT, 1, FUSED, F32OUT>(s, a, r0, c0, out_aligned);
-    else if (nt <= 2) wave_strip<DT, 2, FUSED, F32OUT>(s, a, r0, c0, out_aligned);
-    else if (nt <= 4) wave_strip<DT, 4, FUSED, F32OUT>(s, a, r0, c0, out_aligned);
-    else if (nt <= 8) wave_strip<DT, 8, FUSED, F32OUT>(s, a, r0, c0, out_aligned);
-    else wave_strip<DT, 16, FUSED, F32OUT>(s, a, r0, c0, out_aligned);
+__device__ __forceinline__ void wave_strip_dispatch(int nt, const Seg &s, const RunArgs &a, int r0, int c0) {
+    if (nt <= 1) wave_strip<DT, 1, FUSED, F32OUT>(s, a, r0, c0);
+    else if (nt <= 2) wave_strip<DT, 2, FUSED, F32OUT>(s, a, r0, c0);
+    else if (nt <= 4) wave_strip<DT, 4, FUSED, F32OUT>(s, a, r0, c0);
+    else if (nt <= 8) wave_strip<DT, 8, FUSED, F32OUT>(s, a, r0, c0);
+    else wave_strip<DT, 16, FUSED, F32OUT>(s, a, r0, c0);
 }
 
 __device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
@@ -404,107 +401,180 @@ __device__ __forceinline__ float exchange_row_stats(float (*sM)[16], float (*sL)
     return mine * ginv;
 }
 
-// ------------------------------------------------------------------ kernels
-// Three kernels share one plan: wave_items_kernel (packs, strips / GEMM pieces
-// and the element-wise fallback; wavefronts never synchronise), split_kernel
-// (256 < N <= 4096) and wide_kernel (N > 4096), the latter two with one
-// 16-wave workgroup per strip.  Each loops `for (item = first; item < total;
-// item += stride)`, with the total read from the plan, so any grid size is
-// correct: a grid that covers the items gives one item per wavefront or
-// workgroup and leaves balancing to the hardware dispatcher, a smaller grid
-// strides.
-constexpr int kItemThreads = 256;
-constexpr int kItemWaves = kItemThreads / 64;
+// ------------------------------------------------------ LDS-staged strips
+// All strips of one segment need the same B_g.  The workgroup copies it into
+// LDS once, already in MFMA operand order, with direct global->LDS loads (no
+// registers in between): block (kstep, tile) is the 1 KiB that the 64 lanes of
+// a wavefront feed to one MFMA -- lane i's 16 bytes (row i%16 of the tile, eight
+// k-values of group i/16) sit at byte 16*i.  Reading a block back is therefore
+// one ds_read_b128 per lane at consecutive addresses: conflict-free by
+// construction, no padding or swizzle to compute.  Segments whose B_g exceeds
+// the LDS window are walked in K slabs.
+constexpr int kLdsBlockBytes = 1024;
 
-__device__ __forceinline__ bool plan_matches(PlanHeader *hdr, const RunArgs &a) {
-    if (hdr->magic == kPlanMagic && hdr->kind == 0 && hdr->bad_segments == 0 && hdr->Dm1 == a.Dm1 &&
-        hdr->Dm2 == a.Dm2 && hdr->Dout == a.Dout)
-        return true;
-    if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&hdr->run_errors, 1);
-    return false;
-}
+template <int DT, int NT, bool FUSED, bool F32OUT>
+__device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, unsigned char *lds, int lds_blocks,
+                                                int r0, bool active, int wave, int nwaves) {
+    const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
+    const int K = s.K, N = s.N;
+    const int nt = (N + 15) >> 4;                 // tiles that exist (<= NT)
+    const int nks_total = (K + 31) >> 5;
+    const int slab_ks = max(1, lds_blocks / nt);  // k-steps per LDS fill
+    const SegRes res = make_res(s, a.A, a.B);
+    const int voff = (l16 * K + q * 8) * 2;
+    const int a_soff = r0 * K * 2;
+    const uint16_t *bseg = (const uint16_t *)a.B + s.b;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    f32x4 acc[kMaxTiles];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-// Element-wise path over whole work-item lists: the plan's slow strips always,
-// and every other list too when the launch itself rules out the 16-byte loads
-// (transposed layouts, unaligned base pointers or head strides).
-template <int DT, bool FUSED>
-__device__ __attribute__((noinline)) void generic_phase(const RunArgs &a, bool everything, int64_t gw, int64_t nw) {
-    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const int nseg = hdr->nseg;
-    const PlanRO pv = plan_ro(a.plan, nseg);
-    const int kinds[5] = {kPfxSlow, kPfxPack, FUSED ? kPfxStrip : kPfxGemm, kPfxSplit, kPfxWide};
-    const int nkinds = everything ? (FUSED ? 5 : 3) : 1;
-    for (int ki = 0; ki < nkinds; ++ki) {
-        const int kind = kinds[ki];
-        const int64_t per_head = hdr->totals[kind];
-        const ConstI32 pfx = pv.pfx[kind];
-        for (int64_t it = gw; it < per_head * a.H; it += nw) {
-            const int64_t h = it / per_head;
-            const int i = (int)(it - h * per_head);
-            const int g = prefix_search(pfx, nseg, i);
-            const int local = i - pfx[g];
-            if (kind == kPfxPack) {
-                const int len = pv.recs[g].packLen;
-                for (int j = 0; j < len; ++j) {
-                    const Seg s = load_seg(pv, g + j, h, a);
-                    generic_seg_rows<DT, FUSED>(s, a, 0, s.M, 0, s.N);
+    for (int ks0 = 0; ks0 < nks_total; ks0 += slab_ks) {
+        const int nks = min(slab_ks, nks_total - ks0);
+        if (ks0 > 0) __syncthreads();             // everyone is done reading the previous slab
+        for (int b = wave; b < nt * nks; b += nwaves) {
+            const int t = b % nt, ks = ks0 + b / nt;
+            const int row = min(t * 16 + l16, N - 1);   // ragged last tile: repeat the last row (masked later)
+            int kk = ks * 32 + q * 8;
+            kk = kk < K ? kk : 0;                        // ragged last k-step: any valid address (zeroed at use)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(bseg + (int64_t)row * K + kk),
+                (__attribute__((address_space(3))) void *)(lds + b * kLdsBlockBytes), 16, 0, 0);
+        }
+        u32x4 af = active ? __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + ks0 * 64, 0) : zero;
+        __builtin_amdgcn_s_waitcnt(0);            // this wavefront's LDS fills have landed
+        __syncthreads();
+        if (active) {
+            for (int ksi = 0; ksi < nks; ++ksi) {
+                const int ks = ks0 + ksi;
+                u32x4 af_next = zero;
+                if (ksi + 1 < nks) af_next = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + (ks + 1) * 64, 0);
+                const bool ragged = (ks + 1) * 32 > K;
+                const bool live = ks * 32 + q * 8 < K;
+                if (ragged) af = live ? af : zero;
+                const unsigned char *blk = lds + (ksi * nt) * kLdsBlockBytes + lane * 16;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (t < nt) {
+                        u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + t * kLdsBlockBytes);
+                        if (ragged) bf = live ? bf : zero;
+                        acc[t] = Elem<DT>::mfma(bf, af, acc[t]);
+                    }
                 }
-                continue;
+                af = af_next;
             }
-            const Seg s = load_seg(pv, g, h, a);
-            int r0 = local * kStripRows, c0 = 0, c1 = s.N;
-            if (kind == kPfxGemm) {
-                const int chunks = (s.N + kWaveCols - 1) / kWaveCols;
-                r0 = (local / chunks) * kStripRows; c0 = (local % chunks) * kWaveCols; c1 = c0 + kWaveCols;
-            }
-            generic_seg_rows<DT, FUSED>(s, a, r0, r0 + kStripRows, c0, c1);
         }
     }
+    if (!active) return;
+    float factor = 1.f;
+    if (FUSED) {
+        float c = a.scale * kLog2e;
+        if (c < 0.f) { negate<NT>(acc); c = -c; }
+        float m, l;
+        local_softmax<NT>(acc, N, 0, c, m, l);
+        factor = 1.f / l;
+    }
+    store_rows<DT, NT, F32OUT>(acc, s, a.out, r0, 0, factor);
 }
 
 template <int DT, bool FUSED, bool F32OUT>
-__global__ __launch_bounds__(kItemThreads, 4) void wave_items_kernel(RunArgs a) {
-    PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
-    if (!plan_matches(hdr, a)) return;
-    const int nseg = hdr->nseg;
-    const PlanRO pv = plan_ro(a.plan, nseg);
+__device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, const RunArgs &a, unsigned char *lds,
+                                                         int lds_blocks, int r0, bool active, int wave, int nwaves) {
+    if (nt <= 1) strips_from_lds<DT, 1, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 2) strips_from_lds<DT, 2, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 4) strips_from_lds<DT, 4, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 8) strips_from_lds<DT, 8, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else strips_from_lds<DT, 16, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+}
+
+// ------------------------------------------------------------------ kernels
+// segment_kernel   grid (segment, head, z): one workgroup per segment and head;
+//                  its wavefronts take the segment's 16-row strips (N <= 256),
+//                  the pack it leads, or its rows on the element-wise path.
+//                  No search: the block index is the segment.
+// gemm_large_kernel  GEMM only, N > 256: one wavefront per 16 x 256 piece, found
+//                  by a search in the scanned piece counts.
+// split_kernel / wide_kernel  fused, N > 256: one 16-wave workgroup per strip.
+// The list kernels loop `for (item = first; item < total; item += stride)` with
+// the total read from the plan, so any grid size is correct.
+constexpr int kSegWaves = 4;
+constexpr int kSegThreads = 64 * kSegWaves;
+
+// The header fields every kernel checks, fetched as one batch of scalar loads
+// (no branch between them) before anything depends on them.
+struct HeaderCheck {
+    int nseg;
+    bool ok;
+};
+__device__ __forceinline__ HeaderCheck check_header(const RunArgs &a) {
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+    const uint32_t magic = hdr->magic;
+    const int nseg = hdr->nseg, kind = hdr->kind, bad = hdr->bad_segments;
+    const int64_t d1 = hdr->Dm1, d2 = hdr->Dm2, dO = hdr->Dout;
+    HeaderCheck r;
+    r.nseg = nseg;
+    r.ok = (magic == kPlanMagic) & (kind == 0) & (bad == 0) & (d1 == a.Dm1) & (d2 == a.Dm2) & (dO == a.Dout);
+    return r;
+}
+__device__ __forceinline__ void report_mismatch(const RunArgs &a) {
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+        atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+}
+
+template <int DT, bool FUSED, bool F32OUT>
+__global__ __launch_bounds__(kSegThreads, 4) void segment_kernel(RunArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    const HeaderCheck hc = check_header(a);
+    const int g = blockIdx.x;
+    if (!hc.ok) { report_mismatch(a); return; }
+    if (g >= hc.nseg) return;
+    const PlanRO pv = plan_ro(a.plan, hc.nseg);
+    const int64_t h = blockIdx.y;
     const int wave = uniform((int)(threadIdx.x >> 6));
-    const int64_t gw = (int64_t)blockIdx.x * kItemWaves + wave;
-    const int64_t nw = (int64_t)gridDim.x * kItemWaves;
-    const bool out_aligned = ((uintptr_t)a.out & 15) == 0;
+    const int first = blockIdx.z * kSegWaves + wave, stride = gridDim.z * kSegWaves;
+    const Seg s = load_seg(pv, g, h, a);
+    const int kind = pv.recs[g].kind;
     const bool mfma_ok = (a.flags & kFlagMfmaOk) != 0;
-    if (!mfma_ok || hdr->totals[kPfxSlow] != 0) generic_phase<DT, FUSED>(a, !mfma_ok, gw, nw);
-    if (!mfma_ok) return;
-    {
-        const int64_t per_head = hdr->totals[kPfxPack];
-        const ConstI32 pfx = pv.pfx[kPfxPack];
-        for (int64_t it = gw; it < per_head * a.H; it += nw) {
-            const int64_t h = it / per_head;
-            const int i = (int)(it - h * per_head);
-            const int g = prefix_search(pfx, nseg, i);
-            wave_pack<DT, FUSED, F32OUT>(pv, g, pv.recs[g].packLen, h, a);
-        }
+    if (kind == kSegEmpty) return;
+    if (!mfma_ok || kind == kSegSlow) {
+        // Element-wise path.  With MFMA ruled out for the whole launch this also
+        // covers the segments the list kernels would have taken.
+        for (int r = first; r < s.M; r += stride) generic_seg_rows<DT, FUSED>(s, a, r, r + 1, 0, s.N);
+        return;
     }
-    {
-        const int kind = FUSED ? kPfxStrip : kPfxGemm;
-        const int64_t per_head = hdr->totals[kind];
-        const ConstI32 pfx = pv.pfx[kind];
-        for (int64_t it = gw; it < per_head * a.H; it += nw) {
-            const int64_t h = it / per_head;
-            const int i = (int)(it - h * per_head);
-            const int g = prefix_search(pfx, nseg, i);
-            const int local = i - pfx[g];
-            const Seg s = load_seg(pv, g, h, a);
-            int r0, c0;
-            if (FUSED) {
-                r0 = local * kStripRows; c0 = 0;
-            } else {
-                const int chunks = (s.N + kWaveCols - 1) / kWaveCols;
-                r0 = (local / chunks) * kStripRows; c0 = (local % chunks) * kWaveCols;
-            }
-            const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
-            wave_strip_dispatch<DT, FUSED, F32OUT>(nt, s, a, r0, c0, out_aligned);
+    if (kind == kSegStrip) {
+        // One strip per wavefront; blockIdx.z selects the group of kSegWaves strips.
+        const int strips = (s.M + kStripRows - 1) / kStripRows;
+        const int nt = (s.N + 15) >> 4;
+        for (int base = blockIdx.z * kSegWaves; base < strips; base += gridDim.z * kSegWaves) {
+            if (base != (int)blockIdx.z * kSegWaves) __syncthreads();    // LDS is refilled for the next group
+            const int strip = base + wave;
+            strips_from_lds_dispatch<DT, FUSED, F32OUT>(nt, s, a, lds, a.lds_blocks, strip * kStripRows,
+                                                        strip < strips, wave, kSegWaves);
         }
+    } else if (kind == kSegPackLead) {
+        if (first == 0) wave_pack<DT, FUSED, F32OUT>(pv, g, pv.recs[g].packLen, h, a);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kSegThreads, 4) void gemm_large_kernel(RunArgs a) {
+    const HeaderCheck hc = check_header(a);
+    if (!hc.ok | !(a.flags & kFlagMfmaOk)) return;     // the segment kernel reports and covers these cases
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+    const PlanRO pv = plan_ro(a.plan, hc.nseg);
+    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int per_head = (int)hdr->totals[kPfxGemm];
+    const ConstI32 pfx = pv.pfx[kPfxGemm];
+    const int64_t h = blockIdx.y;
+    for (int i = blockIdx.x * kSegWaves + wave; i < per_head; i += gridDim.x * kSegWaves) {
+        const int g = prefix_search(pfx, hc.nseg, i);
+        const int local = i - pfx[g];
+        const Seg s = load_seg(pv, g, h, a);
+        const int chunks = (s.N + kWaveCols - 1) / kWaveCols;
+        const int r0 = (local / chunks) * kStripRows, c0 = (local % chunks) * kWaveCols;
+        const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
+        wave_strip_dispatch<DT, false, false>(nt, s, a, r0, c0);
     }
 }
 
@@ -515,25 +585,23 @@ __global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
     // never overwrites statistics its neighbours are still reading.
     __shared__ float sM[2][kWavesPerGroup][16];
     __shared__ float sL[2][kWavesPerGroup][16];
-    PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
-    if (!(a.flags & kFlagMfmaOk) || !plan_matches(hdr, a)) return;
-    const int nseg = hdr->nseg;
-    const PlanRO pv = plan_ro(a.plan, nseg);
+    const HeaderCheck hc = check_header(a);
+    if (!hc.ok | !(a.flags & kFlagMfmaOk)) return;
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+    const PlanRO pv = plan_ro(a.plan, hc.nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
-    const bool out_aligned = ((uintptr_t)a.out & 15) == 0;
-    const int64_t per_head = hdr->totals[kPfxSplit];
+    const int per_head = (int)hdr->totals[kPfxSplit];
     const ConstI32 pfx = pv.pfx[kPfxSplit];
+    const int64_t h = blockIdx.y;
     float c = a.scale * kLog2e;
     const bool neg = c < 0.f;
     if (neg) c = -c;
     int xchg = 0;
-    for (int64_t it = blockIdx.x; it < per_head * a.H; it += gridDim.x) {
-        const int64_t h = it / per_head;
-        const int i = (int)(it - h * per_head);
-        const int g = prefix_search(pfx, nseg, i);
+    for (int i = blockIdx.x; i < per_head; i += gridDim.x) {
+        const int g = prefix_search(pfx, hc.nseg, i);
         const int r0 = (i - pfx[g]) * kStripRows;
         const Seg s = load_seg(pv, g, h, a);
-        const SegRes res = make_res<F32OUT ? 4 : 2>(s, a.A, a.B, a.out);
+        const SegRes res = make_res(s, a.A, a.B);
         const int c0 = wave * kWaveCols;
         const int nt = max(0, min(kMaxTiles, (s.N - c0 + 15) >> 4));
         f32x4 acc[kMaxTiles];
@@ -554,11 +622,11 @@ __global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
         ++xchg;
         float gshift, ginv;
         const float factor = exchange_row_stats(sM[buf], sL[buf], wave, m, l, c, gshift, ginv);
-        if (nt > 8) store_rows<DT, 16, F32OUT>(acc, s, res, r0, c0, factor, out_aligned);
-        else if (nt > 4) store_rows<DT, 8, F32OUT>(acc, s, res, r0, c0, factor, out_aligned);
-        else if (nt > 2) store_rows<DT, 4, F32OUT>(acc, s, res, r0, c0, factor, out_aligned);
-        else if (nt > 1) store_rows<DT, 2, F32OUT>(acc, s, res, r0, c0, factor, out_aligned);
-        else if (nt > 0) store_rows<DT, 1, F32OUT>(acc, s, res, r0, c0, factor, out_aligned);
+        if (nt > 8) store_rows<DT, 16, F32OUT>(acc, s, a.out, r0, c0, factor);
+        else if (nt > 4) store_rows<DT, 8, F32OUT>(acc, s, a.out, r0, c0, factor);
+        else if (nt > 2) store_rows<DT, 4, F32OUT>(acc, s, a.out, r0, c0, factor);
+        else if (nt > 1) store_rows<DT, 2, F32OUT>(acc, s, a.out, r0, c0, factor);
+        else if (nt > 0) store_rows<DT, 1, F32OUT>(acc, s, a.out, r0, c0, factor);
     }
 }
 
@@ -568,25 +636,23 @@ template <int DT, bool F32OUT>
 __global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
     __shared__ float sM[2][kWavesPerGroup][16];
     __shared__ float sL[2][kWavesPerGroup][16];
-    PlanHeader *hdr = reinterpret_cast<PlanHeader *>(a.plan);
-    if (!(a.flags & kFlagMfmaOk) || !plan_matches(hdr, a)) return;
-    const int nseg = hdr->nseg;
-    const PlanRO pv = plan_ro(a.plan, nseg);
+    const HeaderCheck hc = check_header(a);
+    if (!hc.ok | !(a.flags & kFlagMfmaOk)) return;
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+    const PlanRO pv = plan_ro(a.plan, hc.nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
-    const bool out_aligned = ((uintptr_t)a.out & 15) == 0;
-    const int64_t per_head = hdr->totals[kPfxWide];
+    const int per_head = (int)hdr->totals[kPfxWide];
     const ConstI32 pfx = pv.pfx[kPfxWide];
+    const int64_t h = blockIdx.y;
     float c = a.scale * kLog2e;
     const bool neg = c < 0.f;
     if (neg) c = -c;
     int xchg = 0;
-    for (int64_t it = blockIdx.x; it < per_head * a.H; it += gridDim.x) {
-        const int64_t h = it / per_head;
-        const int i = (int)(it - h * per_head);
-        const int g = prefix_search(pfx, nseg, i);
+    for (int i = blockIdx.x; i < per_head; i += gridDim.x) {
+        const int g = prefix_search(pfx, hc.nseg, i);
         const int r0 = (i - pfx[g]) * kStripRows;
         const Seg s = load_seg(pv, g, h, a);
-        const SegRes res = make_res<F32OUT ? 4 : 2>(s, a.A, a.B, a.out);
+        const SegRes res = make_res(s, a.A, a.B);
         f32x4 acc[kMaxTiles];
         float run_m = -INFINITY, run_l = 0.f;
         for (int cb = 0; cb < s.N; cb += kSplitCols) {
@@ -617,49 +683,73 @@ __global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
             for (int t = 0; t < kMaxTiles; ++t)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) acc[t][k] = __builtin_amdgcn_exp2f(fmaf(acc[t][k], c, bias));
-            store_rows<DT, kMaxTiles, F32OUT>(acc, s, res, r0, c0, ginv, out_aligned);
+            store_rows<DT, kMaxTiles, F32OUT>(acc, s, a.out, r0, c0, ginv);
         }
     }
 }
 
 // --------------------------------------------------------------------- host
-// Grid sizes.  With a host copy of the plan summary the grids cover the items
-// exactly (capped) and kernels with nothing to do are not launched; without
-// it every kernel is launched with a resident-size grid and strides.
+// With a host copy of the plan summary the grids cover the work exactly and
+// kernels with nothing to do are not launched; without it every kernel is
+// launched with a generous grid and reads the counts from the plan.
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 template <int DT, bool FUSED, bool F32OUT>
-static int launch_set(const RunArgs &args, const ba_plan_info *info, hipStream_t stream) {
+static int launch_set(const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
+    if (args.H > 65535) return BA_ERR_UNSUPPORTED;      // heads ride on gridDim.y
     const int cus = device_cu_count();
-    const int64_t cap = (int64_t)cus * 64;
-    int64_t g_items = (int64_t)cus * 8, g_split = cus, g_wide = cus;
+    const bool mfma_ok = args.flags & kFlagMfmaOk;
+    const unsigned H = (unsigned)args.H;
+    // segment kernel: z spreads the 16-row strips (or rows) of the largest segment over workgroups
+    int64_t z = 4;
+    bool seg_work = true;
+    int64_t g_gemm = (int64_t)cus * 8, g_split = (int64_t)cus * 4, g_wide = (int64_t)cus * 4;
     if (info) {
-        const bool mfma_ok = args.flags & kFlagMfmaOk;
-        int64_t wave_items = (FUSED ? info->strip_items : info->gemm_items) + info->pack_items + info->slow_items;
-        if (!mfma_ok && FUSED) wave_items += info->split_items + info->wide_items;
-        g_items = std::min(cap, ceil_div(wave_items * args.H, kItemWaves));
-        g_split = mfma_ok ? std::min(cap, info->split_items * args.H) : 0;
-        g_wide = mfma_ok ? std::min(cap, info->wide_items * args.H) : 0;
+        nseg = info->nseg;
+        const int64_t units = mfma_ok && info->slow_items == 0 ? ceil_div(std::min<int64_t>(info->max_M, 256), kStripRows)
+                                                                 : std::min<int64_t>(info->max_M, 4096);
+        z = std::max<int64_t>(1, std::min<int64_t>(64, ceil_div(units, kSegWaves)));
+        seg_work = !mfma_ok || info->strip_items + info->pack_items + info->slow_items > 0;
+        g_gemm = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, ceil_div(info->gemm_items, kSegWaves)) : 0;
+        g_split = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, info->split_items) : 0;
+        g_wide = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, info->wide_items) : 0;
     }
-    if (g_items > 0)
-        hipLaunchKernelGGL((wave_items_kernel<DT, FUSED, F32OUT>), dim3((unsigned)g_items), dim3(kItemThreads), 0,
-                           stream, args);
+    if (nseg > 0 && seg_work) {
+        // LDS window for B_g: whole B_g of the largest strip-class segment if known, else 32 KiB.
+        RunArgs seg_args = args;
+        int64_t blocks = 32;
+        if (info) {
+            const int64_t nt = ceil_div(std::min<int64_t>(std::max<int64_t>(info->max_N, 1), kWaveCols), 16);
+            const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
+            blocks = std::max<int64_t>(nt, std::min<int64_t>(nt * nks, 64));
+        }
+        seg_args.lds_blocks = (int)blocks;
+        hipLaunchKernelGGL((segment_kernel<DT, FUSED, F32OUT>), dim3((unsigned)nseg, H, (unsigned)z),
+                           dim3(kSegThreads), (size_t)blocks * kLdsBlockBytes, stream, seg_args);
+    }
+    if (!FUSED && g_gemm > 0)
+        hipLaunchKernelGGL((gemm_large_kernel<DT>), dim3((unsigned)g_gemm, H), dim3(kSegThreads), 0, stream, args);
     if (FUSED && g_split > 0)
-        hipLaunchKernelGGL((split_kernel<DT, F32OUT>), dim3((unsigned)g_split), dim3(kGroupThreads), 0, stream, args);
+        hipLaunchKernelGGL((split_kernel<DT, F32OUT>), dim3((unsigned)g_split, H), dim3(kGroupThreads), 0, stream,
+                           args);
     if (FUSED && g_wide > 0)
-        hipLaunchKernelGGL((wide_kernel<DT, F32OUT>), dim3((unsigned)g_wide), dim3(kGroupThreads), 0, stream, args);
+        hipLaunchKernelGGL((wide_kernel<DT, F32OUT>), dim3((unsigned)g_wide, H), dim3(kGroupThreads), 0, stream,
+                           args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
-int launch_strips(int dtype, int fused, const RunArgs &args, const ba_plan_info *info, hipStream_t stream) {
+int launch_strips(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
+                  hipStream_t stream) {
     const bool f32out = args.flags & kFlagOutF32;
     if (dtype == BA_F16) {
-        if (!fused) return launch_set<0, false, false>(args, info, stream);
-        return f32out ? launch_set<0, true, true>(args, info, stream) : launch_set<0, true, false>(args, info, stream);
+        if (!fused) return launch_set<0, false, false>(args, nseg, info, stream);
+        return f32out ? launch_set<0, true, true>(args, nseg, info, stream)
+                      : launch_set<0, true, false>(args, nseg, info, stream);
     }
     if (dtype == BA_BF16) {
-        if (!fused) return launch_set<1, false, false>(args, info, stream);
-        return f32out ? launch_set<1, true, true>(args, info, stream) : launch_set<1, true, false>(args, info, stream);
+        if (!fused) return launch_set<1, false, false>(args, nseg, info, stream);
+        return f32out ? launch_set<1, true, true>(args, nseg, info, stream)
+                      : launch_set<1, true, false>(args, nseg, info, stream);
     }
     return BA_ERR_UNSUPPORTED;
 }

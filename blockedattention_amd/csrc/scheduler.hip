@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         const bool packed = pack != 0;
         const bool mfma_ok = aligned && !packed;
         int32_t v32[kNumPrefix], t32[kNumPrefix];
-        v32[kPfxGemm] = mfma_ok ? strips * chunks : 0;
+        v32[kPfxGemm] = (mfma_ok && ni > kWaveCols) ? strips * chunks : 0;
         v32[kPfxStrip] = (mfma_ok && ni <= kWaveCols) ? strips : 0;
         v32[kPfxSplit] = (mfma_ok && ni > kWaveCols && ni <= kSplitCols) ? strips : 0;
         v32[kPfxWide] = (mfma_ok && ni > kSplitCols) ? strips : 0;
@@ -198,7 +198,13 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             SegRec rec;
             rec.off1 = o1; rec.off2 = o2; rec.offO = oO;
             rec.M = mi; rec.N = ni; rec.K = ki; rec.packLen = pack > 0 ? pack : 0;
-            rec.pad_[0] = rec.pad_[1] = 0;
+            rec.kind = strips == 0 ? kSegEmpty
+                       : !aligned ? kSegSlow
+                       : pack > 0 ? kSegPackLead
+                       : pack < 0 ? kSegPackFollow
+                       : ni <= kWaveCols ? kSegStrip
+                       : ni <= kSplitCols ? kSegSplit : kSegWide;
+            rec.pad_ = 0;
             pv.recs[g] = rec;
 #pragma unroll
             for (int q = 0; q < kNumPrefix; ++q) pv.pfx[q][g] = base32[q] + v32[q];

@@ -153,7 +153,7 @@ Tensor gemm_launch(const Tensor &mat1, const Tensor &mat2, Schedule &s, bool t1,
     TORCH_CHECK(leading(mat2) == H, "mat1 and mat2 disagree on the number of heads");
     const int dt = dtype_code(mat1, "sparseBlockedGEMM");
     Tensor out = at::empty({H, s.info.Dout}, mat1.options());
-    check_status(ba_varlen_gemm(s.plan.data_ptr(), &s.info, dt, mat1.data_ptr(), mat2.data_ptr(), out.data_ptr(), H,
+    check_status(ba_varlen_gemm(s.plan.data_ptr(), &s.info, s.info.nseg, dt, mat1.data_ptr(), mat2.data_ptr(), out.data_ptr(), H,
                                 s.info.Dm1, s.info.Dm2, s.info.Dout, t1, t2, current_stream(mat1)),
                  "ba_varlen_gemm");
     return out;
@@ -205,7 +205,7 @@ public:
         const int64_t H = leading(src);
         const int dt = dtype_code(src, "sparseBlockedSoftmax");
         Tensor out = at::empty({H, s.info.Dout}, src.options());
-        check_status(ba_blocked_softmax(s.plan.data_ptr(), &s.info, dt, src.data_ptr(), out.data_ptr(), H,
+        check_status(ba_blocked_softmax(s.plan.data_ptr(), &s.info, s.info.nseg, dt, src.data_ptr(), out.data_ptr(), H,
                                         s.info.Dout, (float)scale, current_stream(src)),
                      "ba_blocked_softmax");
         ctx->save_for_backward({out, s.accumOut, s.M, s.N});
@@ -221,7 +221,8 @@ public:
         Schedule s = schedule_softmax(grad, saved[2], saved[3], saved[1]);
         const int64_t H = leading(y);
         Tensor dx = at::empty_like(y);
-        check_status(ba_blocked_softmax_backward(s.plan.data_ptr(), &s.info, dtype_code(y, "softmax backward"),
+        check_status(ba_blocked_softmax_backward(s.plan.data_ptr(), &s.info, s.info.nseg,
+                                                 dtype_code(y, "softmax backward"),
                                                  y.data_ptr(), grad.data_ptr(), dx.data_ptr(), H, s.info.Dout,
                                                  (float)ctx->saved_data["scale"].toDouble(), current_stream(y)),
                      "ba_blocked_softmax_backward");
@@ -263,7 +264,7 @@ Tensor sparseBlockedGEMMSoftmax_op(const Tensor &mat1, const Tensor &mat2, const
     const int64_t H = leading(mat1);
     TORCH_CHECK(leading(mat2) == H, "mat1 and mat2 disagree on the number of heads");
     Tensor out = at::empty({H, s.info.Dout}, out_fp32 ? mat1.options().dtype(at::kFloat) : mat1.options());
-    check_status(ba_gemm_softmax(s.plan.data_ptr(), &s.info, dtype_code(mat1, "fused"), mat1.data_ptr(),
+    check_status(ba_gemm_softmax(s.plan.data_ptr(), &s.info, s.info.nseg, dtype_code(mat1, "fused"), mat1.data_ptr(),
                                  mat2.data_ptr(), out.data_ptr(), out_fp32 ? BA_F32 : dtype_code(mat1, "fused"), H,
                                  s.info.Dm1, s.info.Dm2, s.info.Dout, (float)scale, current_stream(mat1)),
                  "ba_gemm_softmax");

@@ -106,7 +106,8 @@ int ba_plan_softmax(void *plan, size_t plan_bytes, int64_t nseg,
  * call).  Returns BA_ERR_BAD_METADATA if the scheduler rejected any segment
  * or a kernel refused to run against the plan.
  *
- * The compute entry points below take the summary back as `info` (a HOST
+ * The compute entry points below take `nseg` (the segment count the plan was
+ * built for; it sizes the launch grids) and the summary as `info` (a HOST
  * pointer, may be NULL).  With it they launch exactly the kernels the plan has
  * work for, with grids that cover the work; without it they launch every
  * kernel with a resident-size grid and let the kernels read the counts from
@@ -124,7 +125,7 @@ int ba_plan_read(const void *plan, ba_plan_info *host_info, ba_stream_t stream);
  * layouts (spBlkGEMM.cu:292-329, 363-400).  dtype: BA_F16, BA_BF16 (MFMA,
  * fp32 accumulate) or BA_F32.
  */
-int ba_varlen_gemm(void *plan, const ba_plan_info *info, int dtype, const void *A, const void *B, void *out,
+int ba_varlen_gemm(void *plan, const ba_plan_info *info, int64_t nseg, int dtype, const void *A, const void *B, void *out,
                    int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
                    int transpose1, int transpose2, ba_stream_t stream);
 
@@ -134,7 +135,7 @@ int ba_varlen_gemm(void *plan, const ba_plan_info *info, int dtype, const void *
  * (csrc/sparseBlockedAttention.h:20, csrc/cuda/spBlkSoftmax.cu:375-416);
  * scale = 1.0f reproduces it.  No column limit.  src == dst is allowed.
  */
-int ba_blocked_softmax(void *plan, const ba_plan_info *info, int dtype, const void *src, void *dst,
+int ba_blocked_softmax(void *plan, const ba_plan_info *info, int64_t nseg, int dtype, const void *src, void *dst,
                        int64_t H, int64_t Dsrc, float scale, ba_stream_t stream);
 
 /*
@@ -143,7 +144,7 @@ int ba_blocked_softmax(void *plan, const ba_plan_info *info, int dtype, const vo
  * sparseBlockedSoftmaxBackwardLaunch (csrc/sparseBlockedAttention.h:21,
  * csrc/cuda/spBlkSoftmax.cu:418-459).  dx may alias dy.
  */
-int ba_blocked_softmax_backward(void *plan, const ba_plan_info *info, int dtype, const void *y, const void *dy,
+int ba_blocked_softmax_backward(void *plan, const ba_plan_info *info, int64_t nseg, int dtype, const void *y, const void *dy,
                                 void *dx, int64_t H, int64_t Dsrc, float scale, ba_stream_t stream);
 
 /*
@@ -154,7 +155,7 @@ int ba_blocked_softmax_backward(void *plan, const ba_plan_info *info, int dtype,
  * only the two separate launchers above) and takes a plan from ba_plan_gemm.
  * out_dtype: the operand dtype, or BA_F32 for fp32 probabilities.
  */
-int ba_gemm_softmax(void *plan, const ba_plan_info *info, int dtype, const void *A, const void *B, void *out,
+int ba_gemm_softmax(void *plan, const ba_plan_info *info, int64_t nseg, int dtype, const void *A, const void *B, void *out,
                     int out_dtype, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout, float scale,
                     ba_stream_t stream);
 

@@ -46,11 +46,11 @@ def test_argument_errors_are_reported_without_a_device():
     assert lib.ba_plan_gemm(p, 60000, 4, 0, null, null, null, null, null, null, null) == 1       # lists missing
     assert lib.ba_plan_gemm(p, 60000, -1, 0, null, null, null, null, null, null, null) == 1      # negative count
     assert lib.ba_plan_read(null, None, null) == 1
-    assert lib.ba_varlen_gemm(null, None, 0, null, null, null, 1, 1, 1, 1, 0, 0, null) == 1
-    assert lib.ba_varlen_gemm(p, None, 0, null, null, null, -1, 1, 1, 1, 0, 0, null) == 1
-    assert lib.ba_gemm_softmax(p, None, 2, p, p, p, 2, 1, 8, 8, 1, 1.0, null) == 3                # fp32 operands
-    assert lib.ba_gemm_softmax(p, None, 0, p, p, p, 1, 1, 8, 8, 1, 1.0, null) == 3                # f16 in, bf16 out
-    assert lib.ba_blocked_softmax(null, None, 0, null, null, 1, 1, 1.0, null) == 1
+    assert lib.ba_varlen_gemm(null, None, 1, 0, null, null, null, 1, 1, 1, 1, 0, 0, null) == 1
+    assert lib.ba_varlen_gemm(p, None, 1, 0, null, null, null, -1, 1, 1, 1, 0, 0, null) == 1
+    assert lib.ba_gemm_softmax(p, None, 1, 2, p, p, p, 2, 1, 8, 8, 1, 1.0, null) == 3                # fp32 operands
+    assert lib.ba_gemm_softmax(p, None, 1, 0, p, p, p, 1, 1, 8, 8, 1, 1.0, null) == 3                # f16 in, bf16 out
+    assert lib.ba_blocked_softmax(null, None, 1, 0, null, null, 1, 1, 1.0, null) == 1
     # empty work is not an error and launches nothing
-    assert lib.ba_varlen_gemm(p, None, 0, null, null, null, 0, 0, 0, 0, 0, 0, null) == 0
-    assert lib.ba_blocked_softmax(p, None, 0, null, null, 4, 0, 1.0, null) == 0
+    assert lib.ba_varlen_gemm(p, None, 1, 0, null, null, null, 0, 0, 0, 0, 0, 0, null) == 0
+    assert lib.ba_blocked_softmax(p, None, 1, 0, null, null, 4, 0, 1.0, null) == 0

@@ -101,7 +101,7 @@ def test_unaligned_base_pointers_and_odd_head_stride(dev):
     M2, N2, K2 = [6, 3], [10, 5], [8, 4]
     A2, B2 = random_operands(M2, N2, K2, 3, torch.bfloat16, seed=6)
     plan2 = make_plan(dev, M2, N2, K2)
-    assert (plan2.info.Dm1, plan2.info.Dm2, plan2.info.Dout, plan2.info.gemm_items) == (60, 100, 75, 1)
+    assert (plan2.info.Dm1, plan2.info.Dm2, plan2.info.Dout, plan2.info.strip_items) == (60, 100, 75, 1)
     out2 = torch.empty((3, 75), dtype=torch.bfloat16, device=dev)
     capi.varlen_gemm(plan2, A2.to(dev), B2.to(dev), out2, 3, 60, 100, 75)
     assert_scores_close(out2, oracle.per_segment_torch(A2, B2, M2, N2, K2, want="scores"), "odd head stride")

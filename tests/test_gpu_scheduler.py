@@ -36,7 +36,7 @@ def expected_items(M, N, K):
                 i += 1
     ok = aligned & (pack == 0)
     return {
-        "gemm_items": int((strips * -(-N // 256))[ok].sum()),
+        "gemm_items": int((strips * -(-N // 256))[ok & (N > 256)].sum()),
         "strip_items": int(strips[ok & (N <= 256)].sum()),
         "split_items": int(strips[ok & (N > 256) & (N <= 4096)].sum()),
         "wide_items": int(strips[ok & (N > 4096)].sum()),
