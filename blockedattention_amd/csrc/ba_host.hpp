@@ -24,6 +24,7 @@ struct RunArgs {
     float scale;
     int flags;
     int lds_blocks;   // 1 KiB operand blocks of dynamic LDS given to the segment kernel
+    int nseg;         // segment count the plan was built for (checked against the plan)
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,

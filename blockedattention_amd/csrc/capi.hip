@@ -101,10 +101,10 @@ __attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_p
                                                           const void *A, const void *B, void *out, int64_t H,
                                                           int64_t Dm1, int64_t Dm2, int64_t Dout, int transpose1,
                                                           int transpose2, ba_stream_t stream) {
-    if (!plan || nseg < 0 || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (!plan || nseg < 0 || nseg > (int64_t(1) << 30) || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
     if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
     if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0, 0};
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0, 0, (int)nseg};
     if (transpose1) args.flags |= kFlagTranspose1;
     if (transpose2) args.flags |= kFlagTranspose2;
     args.flags |= mfma_flag(args);
@@ -138,12 +138,12 @@ __attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_
                                                            const void *A, const void *B, void *out, int out_dtype,
                                                            int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
                                                            float scale, ba_stream_t stream) {
-    if (!plan || nseg < 0 || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (!plan || nseg < 0 || nseg > (int64_t(1) << 30) || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
     if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
     if (out_dtype != dtype && out_dtype != BA_F32) return BA_ERR_UNSUPPORTED;
     if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
     if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0};
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, (int)nseg};
     args.flags |= mfma_flag(args);
     if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
     return launch_strips(dtype, 1, args, nseg, info, (hipStream_t)stream);

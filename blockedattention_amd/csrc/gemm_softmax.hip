@@ -163,24 +163,53 @@ __device__ __forceinline__ void stage_scores(f32x4 (&acc)[kMaxTiles], const Seg 
 }
 
 // ------------------------------------------------------------ local softmax
-// In: raw scores.  Out: acc = exp2((s - m) * c) for this wavefront's columns
-// (0 for columns past N), m = the row maximum over these columns (same in the
-// four lanes of a row), l = the row sum of acc.  c = scale * log2(e) >= 0.
-// m_shift (= m, or 0 when m is -inf) is what was subtracted.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;   // one instruction for two new elements; fmaxf() would add a canonicalising max per operand
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Brings raw scores into the form the softmax below takes: the multiplier c =
+// scale * log2(e) made non-negative (scores negated for a negative scale, set
+// to zero for a zero scale, where every probability is 1/N), and the columns of
+// the ragged last tile that lie past N set to -inf, so that no later step needs
+// a column mask.  nt = tiles that exist for this wavefront (<= NT).
 template <int NT>
-__device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int N, int c0, float c, float &m,
-                                              float &l) {
-    const int q = lane_id() >> 4;
+__device__ __forceinline__ void prepare_scores(f32x4 (&acc)[kMaxTiles], int nt, int N, int c0, float &c) {
+    if (c < 0.f) {
+        c = -c;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = -acc[t];
+    } else if (c == 0.f) {
+        c = 1.f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int last = nt - 1;
+    const int rem = N - c0 - last * 16;          // columns of the last tile, 1..16
+    if (rem < 16) {
+        const int q4 = (lane_id() >> 4) * 4;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (t == last) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[t][i] = (q4 + i < rem) ? acc[t][i] : -INFINITY;
+            }
+        }
+    }
+}
+
+// In: prepared scores.  Out: acc = exp2((s - m) * c) for this wavefront's
+// tiles, m = the row maximum over them (the same in the four lanes of a row),
+// l = the row sum of acc.
+template <int NT>
+__device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int nt, float c, float &m, float &l) {
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int col = c0 + t * 16 + q * 4;
-        if (c0 + t * 16 + 16 <= N) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) mx = fmaxf(mx, acc[t][i]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) mx = (col + i < N) ? fmaxf(mx, acc[t][i]) : mx;
+        if (t < nt) {
+            mx = max3(mx, acc[t][0], acc[t][1]);
+            mx = max3(mx, acc[t][2], acc[t][3]);
         }
     }
     mx = quad_column_max(mx);
@@ -189,18 +218,10 @@ __device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int N, in
     float sum = 0.f;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int col = c0 + t * 16 + q * 4;
-        if (c0 + t * 16 + 16 <= N) {
+        if (t < nt) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float p = __builtin_amdgcn_exp2f(fmaf(acc[t][i], c, bias));
-                acc[t][i] = p;
-                sum += p;
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float p = (col + i < N) ? __builtin_amdgcn_exp2f(fmaf(acc[t][i], c, bias)) : 0.f;
                 acc[t][i] = p;
                 sum += p;
             }
@@ -215,77 +236,77 @@ __device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int N, in
 // columns are consecutive in memory and go out as ONE 8-byte (16-bit output)
 // or 16-byte (fp32 output) store whatever the address: row starts are only
 // element-aligned (odd N), and the memory pipeline takes vector stores at any
-// element alignment.  Only the ragged last tile of a row falls back to
-// element stores.
+// element alignment.  Only the ragged last tile of a row uses element stores.
 typedef u32x2 __attribute__((aligned(2))) u32x2_unaligned;
 typedef f32x4 __attribute__((aligned(4))) f32x4_unaligned;
 
-template <int DT, int NT, bool F32OUT>
-__device__ __forceinline__ void store_rows(const f32x4 (&acc)[kMaxTiles], const Seg &s, void *__restrict__ out, int r0,
-                                           int c0, float factor) {
-    const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
-    const int r = r0 + l16;
-    if (r >= s.M) return;
-    const int64_t e0 = s.o + (int64_t)r * s.N;
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const int col = c0 + t * 16 + q * 4;
-        if (col >= s.N) continue;
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = acc[t][i] * factor;
-        if (F32OUT) {
-            float *o = reinterpret_cast<float *>(out) + e0 + col;
-            if (col + 3 < s.N) {
-                *reinterpret_cast<f32x4_unaligned *>(o) = f32x4{v[0], v[1], v[2], v[3]};
-            } else {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (col + i < s.N) o[i] = v[i];
-            }
+template <int DT, bool F32OUT>
+__device__ __forceinline__ void store_quad(void *__restrict__ out, int64_t e, const f32x4 &v, int valid) {
+    if (F32OUT) {
+        float *o = reinterpret_cast<float *>(out) + e;
+        if (valid >= 4) {
+            *reinterpret_cast<f32x4_unaligned *>(o) = v;
         } else {
-            uint16_t *o = reinterpret_cast<uint16_t *>(out) + e0 + col;
-            if (col + 3 < s.N) {
-                *reinterpret_cast<u32x2_unaligned *>(o) =
-                    u32x2{Elem<DT>::pack2(v[0], v[1]), Elem<DT>::pack2(v[2], v[3])};
-            } else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (col + i < s.N) o[i] = Elem<DT>::from_float(v[i]);
-            }
+            for (int i = 0; i < 4; ++i)
+                if (i < valid) o[i] = v[i];
+        }
+    } else {
+        uint16_t *o = reinterpret_cast<uint16_t *>(out) + e;
+        if (valid >= 4) {
+            *reinterpret_cast<u32x2_unaligned *>(o) = u32x2{Elem<DT>::pack2(v[0], v[1]), Elem<DT>::pack2(v[2], v[3])};
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (i < valid) o[i] = Elem<DT>::from_float(v[i]);
         }
     }
 }
 
-template <int NT> __device__ __forceinline__ void negate(f32x4 (&acc)[kMaxTiles]) {
+template <int DT, int NT, bool F32OUT>
+__device__ __forceinline__ void store_rows(const f32x4 (&acc)[kMaxTiles], int nt, const Seg &s, void *__restrict__ out,
+                                           int r0, int c0, float factor) {
+    const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
+    const int r = r0 + l16;
+    if (r >= s.M) return;
+    const int64_t e0 = s.o + (int64_t)r * s.N + c0 + q * 4;
+    const int last = nt - 1;
+    const int rem = s.N - c0 - last * 16;         // columns of the last tile, 1..16
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = -acc[t];
+    for (int t = 0; t < NT; ++t) {
+        if (t < last || (t == last && rem == 16)) {
+            store_quad<DT, F32OUT>(out, e0 + t * 16, acc[t] * factor, 4);
+        } else if (t == last) {
+            store_quad<DT, F32OUT>(out, e0 + t * 16, acc[t] * factor, rem - q * 4);
+        }
+    }
 }
+
 
 // One wavefront, one strip, everything in registers.
 template <int DT, int NT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void wave_strip(const Seg &s, const RunArgs &a, int r0, int c0) {
+__device__ __forceinline__ void wave_strip(int nt, const Seg &s, const RunArgs &a, int r0, int c0) {
     f32x4 acc[kMaxTiles];
     const SegRes res = make_res(s, a.A, a.B);
     stage_scores<DT, NT>(acc, s, res, r0, c0);
     float factor = 1.f;
     if (FUSED) {
         float c = a.scale * kLog2e;
-        if (c < 0.f) { negate<NT>(acc); c = -c; }
+        prepare_scores<NT>(acc, nt, s.N, c0, c);
         float m, l;
-        local_softmax<NT>(acc, s.N, c0, c, m, l);
+        local_softmax<NT>(acc, nt, c, m, l);
         factor = 1.f / l;
     }
-    store_rows<DT, NT, F32OUT>(acc, s, a.out, r0, c0, factor);
+    store_rows<DT, NT, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
 }
 
 template <int DT, bool FUSED, bool F32OUT>
 __device__ __forceinline__ void wave_strip_dispatch(int nt, const Seg &s, const RunArgs &a, int r0, int c0) {
-    if (nt <= 1) wave_strip<DT, 1, FUSED, F32OUT>(s, a, r0, c0);
-    else if (nt <= 2) wave_strip<DT, 2, FUSED, F32OUT>(s, a, r0, c0);
-    else if (nt <= 4) wave_strip<DT, 4, FUSED, F32OUT>(s, a, r0, c0);
-    else if (nt <= 8) wave_strip<DT, 8, FUSED, F32OUT>(s, a, r0, c0);
-    else wave_strip<DT, 16, FUSED, F32OUT>(s, a, r0, c0);
+    if (nt <= 1) wave_strip<DT, 1, FUSED, F32OUT>(nt, s, a, r0, c0);
+    else if (nt <= 2) wave_strip<DT, 2, FUSED, F32OUT>(nt, s, a, r0, c0);
+    else if (nt <= 4) wave_strip<DT, 4, FUSED, F32OUT>(nt, s, a, r0, c0);
+    else if (nt <= 8) wave_strip<DT, 8, FUSED, F32OUT>(nt, s, a, r0, c0);
+    else wave_strip<DT, 16, FUSED, F32OUT>(nt, s, a, r0, c0);
 }
 
 __device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
@@ -436,7 +457,7 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
             const int t = b % nt, ks = ks0 + b / nt;
             const int row = min(t * 16 + l16, N - 1);   // ragged last tile: repeat the last row (masked later)
             int kk = ks * 32 + q * 8;
-            kk = kk < K ? kk : 0;                        // ragged last k-step: any valid address (zeroed at use)
+            kk = kk < K ? kk : 0;                        // ragged last k-step: valid data, multiplied by zeros
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void *)(bseg + (int64_t)row * K + kk),
                 (__attribute__((address_space(3))) void *)(lds + b * kLdsBlockBytes), 16, 0, 0);
@@ -449,15 +470,14 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
                 const int ks = ks0 + ksi;
                 u32x4 af_next = zero;
                 if (ksi + 1 < nks) af_next = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + (ks + 1) * 64, 0);
-                const bool ragged = (ks + 1) * 32 > K;
-                const bool live = ks * 32 + q * 8 < K;
-                if (ragged) af = live ? af : zero;
+                // Ragged last k-step: lanes whose k-group lies past K feed a zero A fragment
+                // (their B fragment is a repeat of valid row data, see the fill above).
+                if ((ks + 1) * 32 > K) af = (ks * 32 + q * 8 < K) ? af : zero;
                 const unsigned char *blk = lds + (ksi * nt) * kLdsBlockBytes + lane * 16;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
                     if (t < nt) {
-                        u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + t * kLdsBlockBytes);
-                        if (ragged) bf = live ? bf : zero;
+                        const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + t * kLdsBlockBytes);
                         acc[t] = Elem<DT>::mfma(bf, af, acc[t]);
                     }
                 }
@@ -469,12 +489,12 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
     float factor = 1.f;
     if (FUSED) {
         float c = a.scale * kLog2e;
-        if (c < 0.f) { negate<NT>(acc); c = -c; }
+        prepare_scores<NT>(acc, nt, N, 0, c);
         float m, l;
-        local_softmax<NT>(acc, N, 0, c, m, l);
+        local_softmax<NT>(acc, nt, c, m, l);
         factor = 1.f / l;
     }
-    store_rows<DT, NT, F32OUT>(acc, s, a.out, r0, 0, factor);
+    store_rows<DT, NT, F32OUT>(acc, nt, s, a.out, r0, 0, factor);
 }
 
 template <int DT, bool FUSED, bool F32OUT>
@@ -501,20 +521,15 @@ constexpr int kSegWaves = 4;
 constexpr int kSegThreads = 64 * kSegWaves;
 
 // The header fields every kernel checks, fetched as one batch of scalar loads
-// (no branch between them) before anything depends on them.
-struct HeaderCheck {
-    int nseg;
-    bool ok;
-};
-__device__ __forceinline__ HeaderCheck check_header(const RunArgs &a) {
+// (no branch between them).  The segment count comes with the launch, so the
+// addresses of the plan's arrays do not wait for the header either.
+__device__ __forceinline__ bool header_ok(const RunArgs &a) {
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
     const uint32_t magic = hdr->magic;
     const int nseg = hdr->nseg, kind = hdr->kind, bad = hdr->bad_segments;
     const int64_t d1 = hdr->Dm1, d2 = hdr->Dm2, dO = hdr->Dout;
-    HeaderCheck r;
-    r.nseg = nseg;
-    r.ok = (magic == kPlanMagic) & (kind == 0) & (bad == 0) & (d1 == a.Dm1) & (d2 == a.Dm2) & (dO == a.Dout);
-    return r;
+    return (magic == kPlanMagic) & (nseg == a.nseg) & (kind == 0) & (bad == 0) & (d1 == a.Dm1) & (d2 == a.Dm2) &
+           (dO == a.Dout);
 }
 __device__ __forceinline__ void report_mismatch(const RunArgs &a) {
     if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
@@ -524,16 +539,17 @@ __device__ __forceinline__ void report_mismatch(const RunArgs &a) {
 template <int DT, bool FUSED, bool F32OUT>
 __global__ __launch_bounds__(kSegThreads, 4) void segment_kernel(RunArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-    const HeaderCheck hc = check_header(a);
     const int g = blockIdx.x;
-    if (!hc.ok) { report_mismatch(a); return; }
-    if (g >= hc.nseg) return;
-    const PlanRO pv = plan_ro(a.plan, hc.nseg);
+    if (g >= a.nseg) return;
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int64_t h = blockIdx.y;
-    const int wave = uniform((int)(threadIdx.x >> 6));
-    const int first = blockIdx.z * kSegWaves + wave, stride = gridDim.z * kSegWaves;
+    // Header and segment record are fetched together; nothing waits on the header alone.
+    const bool ok = header_ok(a);
     const Seg s = load_seg(pv, g, h, a);
     const int kind = pv.recs[g].kind;
+    if (!ok) { report_mismatch(a); return; }
+    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int first = blockIdx.z * kSegWaves + wave, stride = gridDim.z * kSegWaves;
     const bool mfma_ok = (a.flags & kFlagMfmaOk) != 0;
     if (kind == kSegEmpty) return;
     if (!mfma_ok || kind == kSegSlow) {
@@ -559,16 +575,15 @@ __global__ __launch_bounds__(kSegThreads, 4) void segment_kernel(RunArgs a) {
 
 template <int DT>
 __global__ __launch_bounds__(kSegThreads, 4) void gemm_large_kernel(RunArgs a) {
-    const HeaderCheck hc = check_header(a);
-    if (!hc.ok | !(a.flags & kFlagMfmaOk)) return;     // the segment kernel reports and covers these cases
+    if (!header_ok(a) | !(a.flags & kFlagMfmaOk)) return;     // the segment kernel reports and covers these cases
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const PlanRO pv = plan_ro(a.plan, hc.nseg);
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int per_head = (int)hdr->totals[kPfxGemm];
     const ConstI32 pfx = pv.pfx[kPfxGemm];
     const int64_t h = blockIdx.y;
     for (int i = blockIdx.x * kSegWaves + wave; i < per_head; i += gridDim.x * kSegWaves) {
-        const int g = prefix_search(pfx, hc.nseg, i);
+        const int g = prefix_search(pfx, a.nseg, i);
         const int local = i - pfx[g];
         const Seg s = load_seg(pv, g, h, a);
         const int chunks = (s.N + kWaveCols - 1) / kWaveCols;
@@ -585,20 +600,18 @@ __global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
     // never overwrites statistics its neighbours are still reading.
     __shared__ float sM[2][kWavesPerGroup][16];
     __shared__ float sL[2][kWavesPerGroup][16];
-    const HeaderCheck hc = check_header(a);
-    if (!hc.ok | !(a.flags & kFlagMfmaOk)) return;
+    if (!header_ok(a) | !(a.flags & kFlagMfmaOk)) return;
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const PlanRO pv = plan_ro(a.plan, hc.nseg);
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int per_head = (int)hdr->totals[kPfxSplit];
     const ConstI32 pfx = pv.pfx[kPfxSplit];
     const int64_t h = blockIdx.y;
-    float c = a.scale * kLog2e;
-    const bool neg = c < 0.f;
-    if (neg) c = -c;
+    const float c_raw = a.scale * kLog2e;
+    const float c = c_raw < 0.f ? -c_raw : (c_raw == 0.f ? 1.f : c_raw);   // what prepare_scores leaves
     int xchg = 0;
     for (int i = blockIdx.x; i < per_head; i += gridDim.x) {
-        const int g = prefix_search(pfx, hc.nseg, i);
+        const int g = prefix_search(pfx, a.nseg, i);
         const int r0 = (i - pfx[g]) * kStripRows;
         const Seg s = load_seg(pv, g, h, a);
         const SegRes res = make_res(s, a.A, a.B);
@@ -608,9 +621,10 @@ __global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
         float m = -INFINITY, l = 0.f;
 #define BA_SPLIT_STAGE(NT)                              \
     {                                                   \
+        float cc = c_raw;                               \
         stage_scores<DT, NT>(acc, s, res, r0, c0);      \
-        if (neg) negate<NT>(acc);                       \
-        local_softmax<NT>(acc, s.N, c0, c, m, l);       \
+        prepare_scores<NT>(acc, nt, s.N, c0, cc);       \
+        local_softmax<NT>(acc, nt, cc, m, l);           \
     }
         if (nt > 8) BA_SPLIT_STAGE(16)
         else if (nt > 4) BA_SPLIT_STAGE(8)
@@ -622,11 +636,11 @@ __global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
         ++xchg;
         float gshift, ginv;
         const float factor = exchange_row_stats(sM[buf], sL[buf], wave, m, l, c, gshift, ginv);
-        if (nt > 8) store_rows<DT, 16, F32OUT>(acc, s, a.out, r0, c0, factor);
-        else if (nt > 4) store_rows<DT, 8, F32OUT>(acc, s, a.out, r0, c0, factor);
-        else if (nt > 2) store_rows<DT, 4, F32OUT>(acc, s, a.out, r0, c0, factor);
-        else if (nt > 1) store_rows<DT, 2, F32OUT>(acc, s, a.out, r0, c0, factor);
-        else if (nt > 0) store_rows<DT, 1, F32OUT>(acc, s, a.out, r0, c0, factor);
+        if (nt > 8) store_rows<DT, 16, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
+        else if (nt > 4) store_rows<DT, 8, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
+        else if (nt > 2) store_rows<DT, 4, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
+        else if (nt > 1) store_rows<DT, 2, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
+        else if (nt > 0) store_rows<DT, 1, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
     }
 }
 
@@ -636,20 +650,18 @@ template <int DT, bool F32OUT>
 __global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
     __shared__ float sM[2][kWavesPerGroup][16];
     __shared__ float sL[2][kWavesPerGroup][16];
-    const HeaderCheck hc = check_header(a);
-    if (!hc.ok | !(a.flags & kFlagMfmaOk)) return;
+    if (!header_ok(a) | !(a.flags & kFlagMfmaOk)) return;
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const PlanRO pv = plan_ro(a.plan, hc.nseg);
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int per_head = (int)hdr->totals[kPfxWide];
     const ConstI32 pfx = pv.pfx[kPfxWide];
     const int64_t h = blockIdx.y;
-    float c = a.scale * kLog2e;
-    const bool neg = c < 0.f;
-    if (neg) c = -c;
+    const float c_raw = a.scale * kLog2e;
+    const float c = c_raw < 0.f ? -c_raw : (c_raw == 0.f ? 1.f : c_raw);   // what prepare_scores leaves
     int xchg = 0;
     for (int i = blockIdx.x; i < per_head; i += gridDim.x) {
-        const int g = prefix_search(pfx, hc.nseg, i);
+        const int g = prefix_search(pfx, a.nseg, i);
         const int r0 = (i - pfx[g]) * kStripRows;
         const Seg s = load_seg(pv, g, h, a);
         const SegRes res = make_res(s, a.A, a.B);
@@ -658,10 +670,11 @@ __global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
         for (int cb = 0; cb < s.N; cb += kSplitCols) {
             const int c0 = cb + wave * kWaveCols;
             if (c0 >= s.N) continue;
-            float m, l;
+            float m, l, cc = c_raw;
+            const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
             stage_scores<DT, kMaxTiles>(acc, s, res, r0, c0);
-            if (neg) negate<kMaxTiles>(acc);
-            local_softmax<kMaxTiles>(acc, s.N, c0, c, m, l);
+            prepare_scores<kMaxTiles>(acc, nt, s.N, c0, cc);
+            local_softmax<kMaxTiles>(acc, nt, cc, m, l);
             const float nm = fmaxf(run_m, m);
             const float nshift = (nm == -INFINITY) ? 0.f : nm;
             const float f_old = (run_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((run_m - nshift) * c);
@@ -677,13 +690,15 @@ __global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
         for (int cb = 0; cb < s.N; cb += kSplitCols) {
             const int c0 = cb + wave * kWaveCols;
             if (c0 >= s.N) continue;
+            float cc = c_raw;
+            const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
             stage_scores<DT, kMaxTiles>(acc, s, res, r0, c0);
-            if (neg) negate<kMaxTiles>(acc);
+            prepare_scores<kMaxTiles>(acc, nt, s.N, c0, cc);
 #pragma unroll
             for (int t = 0; t < kMaxTiles; ++t)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) acc[t][k] = __builtin_amdgcn_exp2f(fmaf(acc[t][k], c, bias));
-            store_rows<DT, kMaxTiles, F32OUT>(acc, s, a.out, r0, c0, ginv);
+            store_rows<DT, kMaxTiles, F32OUT>(acc, nt, s, a.out, r0, c0, ginv);
         }
     }
 }
