@@ -453,14 +453,16 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
     for (int ks0 = 0; ks0 < nks_total; ks0 += slab_ks) {
         const int nks = min(slab_ks, nks_total - ks0);
         if (ks0 > 0) __syncthreads();             // everyone is done reading the previous slab
-        for (int b = wave; b < nt * nks; b += nwaves) {
-            const int t = b % nt, ks = ks0 + b / nt;
+        for (int t = wave; t < nt; t += nwaves) {       // tile t of every k-step of the slab
             const int row = min(t * 16 + l16, N - 1);   // ragged last tile: repeat the last row (masked later)
-            int kk = ks * 32 + q * 8;
-            kk = kk < K ? kk : 0;                        // ragged last k-step: valid data, multiplied by zeros
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void *)(bseg + (int64_t)row * K + kk),
-                (__attribute__((address_space(3))) void *)(lds + b * kLdsBlockBytes), 16, 0, 0);
+            const uint16_t *brow = bseg + (int64_t)row * K;
+            for (int ksi = 0; ksi < nks; ++ksi) {
+                int kk = (ks0 + ksi) * 32 + q * 8;
+                kk = kk < K ? kk : 0;                    // ragged last k-step: valid data, multiplied by zeros
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(brow + kk),
+                    (__attribute__((address_space(3))) void *)(lds + (ksi * nt + t) * kLdsBlockBytes), 16, 0, 0);
+            }
         }
         u32x4 af = active ? __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + ks0 * 64, 0) : zero;
         __builtin_amdgcn_s_waitcnt(0);            // this wavefront's LDS fills have landed
@@ -497,13 +499,13 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
     store_rows<DT, NT, F32OUT>(acc, nt, s, a.out, r0, 0, factor);
 }
 
-template <int DT, bool FUSED, bool F32OUT>
+template <int DT, bool FUSED, bool F32OUT, int MAXNT>
 __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, const RunArgs &a, unsigned char *lds,
                                                          int lds_blocks, int r0, bool active, int wave, int nwaves) {
     if (nt <= 1) strips_from_lds<DT, 1, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
     else if (nt <= 2) strips_from_lds<DT, 2, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
     else if (nt <= 4) strips_from_lds<DT, 4, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
-    else if (nt <= 8) strips_from_lds<DT, 8, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 8 || MAXNT <= 8) strips_from_lds<DT, 8, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
     else strips_from_lds<DT, 16, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
 }
 
@@ -536,8 +538,11 @@ __device__ __forceinline__ void report_mismatch(const RunArgs &a) {
         atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
 }
 
-template <int DT, bool FUSED, bool F32OUT>
-__global__ __launch_bounds__(kSegThreads, 4) void segment_kernel(RunArgs a) {
+// MAXNT = 8 is the build for batches whose widest segment has N <= 128: half the
+// accumulator registers, twice the resident wavefronts.  The host picks it from
+// the plan summary; without a summary the 16-tile build runs.
+template <int DT, bool FUSED, bool F32OUT, int MAXNT>
+__global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 8 : 4) void segment_kernel(RunArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const int g = blockIdx.x;
     if (g >= a.nseg) return;
@@ -565,7 +570,7 @@ __global__ __launch_bounds__(kSegThreads, 4) void segment_kernel(RunArgs a) {
         for (int base = blockIdx.z * kSegWaves; base < strips; base += gridDim.z * kSegWaves) {
             if (base != (int)blockIdx.z * kSegWaves) __syncthreads();    // LDS is refilled for the next group
             const int strip = base + wave;
-            strips_from_lds_dispatch<DT, FUSED, F32OUT>(nt, s, a, lds, a.lds_blocks, strip * kStripRows,
+            strips_from_lds_dispatch<DT, FUSED, F32OUT, MAXNT>(nt, s, a, lds, a.lds_blocks, strip * kStripRows,
                                                         strip < strips, wave, kSegWaves);
         }
     } else if (kind == kSegPackLead) {
@@ -739,8 +744,14 @@ static int launch_set(const RunArgs &args, int64_t nseg, const ba_plan_info *inf
             blocks = std::max<int64_t>(nt, std::min<int64_t>(nt * nks, 64));
         }
         seg_args.lds_blocks = (int)blocks;
-        hipLaunchKernelGGL((segment_kernel<DT, FUSED, F32OUT>), dim3((unsigned)nseg, H, (unsigned)z),
-                           dim3(kSegThreads), (size_t)blocks * kLdsBlockBytes, stream, seg_args);
+        const dim3 grid((unsigned)nseg, H, (unsigned)z);
+        const size_t lds_bytes = (size_t)blocks * kLdsBlockBytes;
+        if (info && info->max_N <= 128)
+            hipLaunchKernelGGL((segment_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream,
+                               seg_args);
+        else
+            hipLaunchKernelGGL((segment_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream,
+                               seg_args);
     }
     if (!FUSED && g_gemm > 0)
         hipLaunchKernelGGL((gemm_large_kernel<DT>), dim3((unsigned)g_gemm, H), dim3(kSegThreads), 0, stream, args);
