@@ -59,32 +59,55 @@ class Case:
         self.M, self.N, self.K = i64(w.M), i64(w.N), i64(w.K)
         self.acc = [torch.empty(w.nseg + 1, dtype=torch.int64, device=dev) for _ in range(3)]
         self.out = torch.empty((w.heads, w.Dout), dtype=w.dtype, device=dev)
-        self.scores = None
         self.plan = capi.plan_gemm(w.nseg, dev, self.M, self.N, self.K, *self.acc, mode=capi.META_FROM_LISTS)
         self.plan.read()
         self.dev = dev
+        self._bind()
+
+    def _bind(self):
+        """Pre-converted ctypes argument tuples: the timed loops then cost one foreign call per launch."""
+        import ctypes
+        c, w, p = self.capi, self.w, self.plan
+        lib, st = c.load(), c._stream()
+        i64, i32, f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_float
+        code = i32(c.dtype_code(w.dtype))
+        dims = (i64(w.heads), i64(w.Dm1), i64(w.Dm2), i64(w.Dout))
+        self._lib = lib
+        self._a_sched = (p.ptr, ctypes.c_size_t(p.bytes), i64(w.nseg), i32(c.META_FROM_LISTS), c._ptr(self.M),
+                         c._ptr(self.N), c._ptr(self.K), c._ptr(self.acc[0]), c._ptr(self.acc[1]),
+                         c._ptr(self.acc[2]), st)
+        self._a_fused = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.out), code,
+                         *dims, f32(w.scale), st)
+        self.scores = self.torch.empty_like(self.out)
+        self._a_gemm = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.scores),
+                        *dims, i32(0), i32(0), st)
+        self._a_soft = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.scores), c._ptr(self.out), i64(w.heads),
+                        i64(w.Dout), f32(w.scale), st)
+        for st_code, what in ((lib.ba_plan_gemm(*self._a_sched), "ba_plan_gemm"),
+                              (lib.ba_gemm_softmax(*self._a_fused), "ba_gemm_softmax"),
+                              (lib.ba_varlen_gemm(*self._a_gemm), "ba_varlen_gemm"),
+                              (lib.ba_blocked_softmax(*self._a_soft), "ba_blocked_softmax")):
+            c.check(st_code, what)
 
     def schedule(self):
-        c, w, p = self.capi, self.w, self.plan
-        st = c.load().ba_plan_gemm(p.ptr, p.bytes, w.nseg, c.META_FROM_LISTS, c._ptr(self.M), c._ptr(self.N),
-                                   c._ptr(self.K), c._ptr(self.acc[0]), c._ptr(self.acc[1]), c._ptr(self.acc[2]),
-                                   c._stream())
-        c.check(st, "ba_plan_gemm")
+        self._lib.ba_plan_gemm(*self._a_sched)
 
     def fused(self):
-        w = self.w
-        self.capi.gemm_softmax(self.plan, self.A, self.B, self.out, w.heads, w.Dm1, w.Dm2, w.Dout, w.scale)
+        self._lib.ba_gemm_softmax(*self._a_fused)
+
+    def gemm(self):
+        self._lib.ba_varlen_gemm(*self._a_gemm)
+
+    def softmax(self):
+        self._lib.ba_blocked_softmax(*self._a_soft)
 
     def step(self):
-        self.schedule()
-        self.fused()
+        self._lib.ba_plan_gemm(*self._a_sched)
+        self._lib.ba_gemm_softmax(*self._a_fused)
 
     def unfused(self):
-        w = self.w
-        if self.scores is None:
-            self.scores = self.torch.empty_like(self.out)
-        self.capi.varlen_gemm(self.plan, self.A, self.B, self.scores, w.heads, w.Dm1, w.Dm2, w.Dout)
-        self.capi.blocked_softmax(self.plan, self.scores, self.out, w.heads, w.Dout, w.scale)
+        self._lib.ba_varlen_gemm(*self._a_gemm)
+        self._lib.ba_blocked_softmax(*self._a_soft)
 
     def event_us(self, fn, steps, warmup):
         """Average device time of fn over `steps` back-to-back calls, HIP events on the launch stream."""
@@ -148,6 +171,8 @@ class Case:
             "mfma_frac": round(w.flops / k_us * 1e-6 / MFMA_PEAK_TFLOPS, 4),
         }
         if with_unfused:
+            fig["gemm_only_us"] = round(self.event_us(self.gemm, steps, warmup), 3)
+            fig["softmax_only_us"] = round(self.event_us(self.softmax, steps, warmup), 3)
             fig["unfused_pair_us"] = round(self.event_us(self.unfused, steps, warmup), 3)
         return fig
 
@@ -206,7 +231,7 @@ def main():
         "config": {"workload": w.name, "segments": w.nseg, "heads": w.heads, "seed": 0,
                    "flops": w.flops, "pair_bytes": w.pair_bytes()},
         "roofline": {"bound": "hbm", "achieved": fig["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": fig["hbm_frac"], "traffic": None, "kernel": "wave_items_kernel (fused)",
+                     "frac": fig["hbm_frac"], "traffic": None, "kernel": "ba::segment_kernel (fused GEMM+softmax)",
                      "kernel_us": fig["kernel_us"], "mfma_frac": fig["mfma_frac"], "TFLOPs": fig["TFLOPs"]},
         "parity_max_abs_err": worst,
         "detail": fig,
