@@ -432,15 +432,19 @@ __device__ __forceinline__ float exchange_row_stats(float (*sM)[16], float (*sL)
 // construction, no padding or swizzle to compute.  Segments whose B_g exceeds
 // the LDS window are walked in K slabs.
 constexpr int kLdsBlockBytes = 1024;
+// k-steps (of 32) whose A fragments a wavefront keeps in registers: 4 in the 128-register build, 2 in the
+// leaner build (larger K takes more slabs)
+template <int MAXNT> struct SlabSteps { static constexpr int value = MAXNT <= 8 ? 2 : 4; };
 
-template <int DT, int NT, bool FUSED, bool F32OUT>
+template <int DT, int NT, bool FUSED, bool F32OUT, int MAXNT>
 __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, unsigned char *lds, int lds_blocks,
                                                 int r0, bool active, int wave, int nwaves) {
     const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
     const int K = s.K, N = s.N;
     const int nt = (N + 15) >> 4;                 // tiles that exist (<= NT)
+    constexpr int kSlabSteps = SlabSteps<MAXNT>::value;
     const int nks_total = (K + 31) >> 5;
-    const int slab_ks = max(1, lds_blocks / nt);  // k-steps per LDS fill
+    const int slab_ks = max(1, min(kSlabSteps, lds_blocks / nt));  // k-steps per LDS fill
     const SegRes res = make_res(s, a.A, a.B);
     const int voff = (l16 * K + q * 8) * 2;
     const int a_soff = r0 * K * 2;
@@ -453,6 +457,17 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
     for (int ks0 = 0; ks0 < nks_total; ks0 += slab_ks) {
         const int nks = min(slab_ks, nks_total - ks0);
         if (ks0 > 0) __syncthreads();             // everyone is done reading the previous slab
+        // The wavefront's own A fragments of the slab go to registers first, so their
+        // latency runs under the LDS fill and nothing is fetched inside the MFMA loop.
+        u32x4 af[kSlabSteps];
+#pragma unroll
+        for (int ksi = 0; ksi < kSlabSteps; ++ksi) {
+            af[ksi] = zero;
+            if (active && ksi < nks) {
+                const int ks = ks0 + ksi;
+                af[ksi] = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + ks * 64, 0);
+            }
+        }
         for (int t = wave; t < nt; t += nwaves) {       // tile t of every k-step of the slab
             const int row = min(t * 16 + l16, N - 1);   // ragged last tile: repeat the last row (masked later)
             const uint16_t *brow = bseg + (int64_t)row * K;
@@ -464,26 +479,28 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
                     (__attribute__((address_space(3))) void *)(lds + (ksi * nt + t) * kLdsBlockBytes), 16, 0, 0);
             }
         }
-        u32x4 af = active ? __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + ks0 * 64, 0) : zero;
-        __builtin_amdgcn_s_waitcnt(0);            // this wavefront's LDS fills have landed
+        __builtin_amdgcn_s_waitcnt(0);            // this wavefront's loads and LDS fills have landed
         __syncthreads();
         if (active) {
-            for (int ksi = 0; ksi < nks; ++ksi) {
-                const int ks = ks0 + ksi;
-                u32x4 af_next = zero;
-                if (ksi + 1 < nks) af_next = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + (ks + 1) * 64, 0);
-                // Ragged last k-step: lanes whose k-group lies past K feed a zero A fragment
-                // (their B fragment is a repeat of valid row data, see the fill above).
-                if ((ks + 1) * 32 > K) af = (ks * 32 + q * 8 < K) ? af : zero;
-                const unsigned char *blk = lds + (ksi * nt) * kLdsBlockBytes + lane * 16;
+            // Ragged last k-step: lanes whose k-group lies past K feed a zero A fragment
+            // (their B fragment is a repeat of valid row data, see the fill above).
+            if ((ks0 + nks) * 32 > K) {
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    if (t < nt) {
-                        const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + t * kLdsBlockBytes);
-                        acc[t] = Elem<DT>::mfma(bf, af, acc[t]);
+                for (int ksi = 0; ksi < kSlabSteps; ++ksi)
+                    if (ksi == nks - 1) af[ksi] = ((ks0 + ksi) * 32 + q * 8 < K) ? af[ksi] : zero;
+            }
+#pragma unroll
+            for (int ksi = 0; ksi < kSlabSteps; ++ksi) {
+                if (ksi < nks) {
+                    const unsigned char *blk = lds + (ksi * nt) * kLdsBlockBytes + lane * 16;
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        if (t < nt) {
+                            const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + t * kLdsBlockBytes);
+                            acc[t] = Elem<DT>::mfma(bf, af[ksi], acc[t]);
+                        }
                     }
                 }
-                af = af_next;
             }
         }
     }
@@ -502,11 +519,11 @@ __device__ __forceinline__ void strips_from_lds(const Seg &s, const RunArgs &a, 
 template <int DT, bool FUSED, bool F32OUT, int MAXNT>
 __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, const RunArgs &a, unsigned char *lds,
                                                          int lds_blocks, int r0, bool active, int wave, int nwaves) {
-    if (nt <= 1) strips_from_lds<DT, 1, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
-    else if (nt <= 2) strips_from_lds<DT, 2, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
-    else if (nt <= 4) strips_from_lds<DT, 4, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
-    else if (nt <= 8 || MAXNT <= 8) strips_from_lds<DT, 8, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
-    else strips_from_lds<DT, 16, FUSED, F32OUT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    if (nt <= 1) strips_from_lds<DT, 1, FUSED, F32OUT, MAXNT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 2) strips_from_lds<DT, 2, FUSED, F32OUT, MAXNT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 4) strips_from_lds<DT, 4, FUSED, F32OUT, MAXNT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else if (nt <= 8 || MAXNT <= 8) strips_from_lds<DT, 8, FUSED, F32OUT, MAXNT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
+    else strips_from_lds<DT, 16, FUSED, F32OUT, MAXNT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
 }
 
 // ------------------------------------------------------------------ kernels
@@ -539,10 +556,10 @@ __device__ __forceinline__ void report_mismatch(const RunArgs &a) {
 }
 
 // MAXNT = 8 is the build for batches whose widest segment has N <= 128: half the
-// accumulator registers, twice the resident wavefronts.  The host picks it from
+// accumulator registers, half again as many resident wavefronts.  The host picks it from
 // the plan summary; without a summary the 16-tile build runs.
 template <int DT, bool FUSED, bool F32OUT, int MAXNT>
-__global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 8 : 4) void segment_kernel(RunArgs a) {
+__global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kernel(RunArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const int g = blockIdx.x;
     if (g >= a.nseg) return;
