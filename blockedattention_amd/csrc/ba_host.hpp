@@ -12,7 +12,8 @@ enum RunFlags : int {
     kFlagTranspose1 = 1,   // A segments stored K x M
     kFlagTranspose2 = 2,   // B segments stored K x N
     kFlagMfmaOk = 4,       // layouts, base pointers and head strides allow 16-byte operand loads
-    kFlagOutF32 = 8        // fused path writes fp32 probabilities
+    kFlagOutF32 = 8,       // fused path writes fp32 probabilities
+    kFlagFastStrips = 16   // the strip kernel runs in the same call and takes the segments that fit its window
 };
 
 struct RunArgs {

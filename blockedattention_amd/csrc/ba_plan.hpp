@@ -21,6 +21,16 @@ constexpr int kWavesPerGroup = 16;
 constexpr int kSplitCols = kWaveCols * kWavesPerGroup;  // 4096: columns one workgroup keeps in registers
 constexpr int kPackDim = 16;      // a pack of tiny segments fits one 16x16 MFMA tile
 
+// Strip-class segments whose whole B_g fits the strip kernel's LDS window: G =
+// the even tile count covering N, G * ceil(K/32) operand blocks of 1 KiB.
+constexpr int kFastBlocks = 32;
+constexpr int kFastSteps = 4;     // k-steps of 32 whose A fragments a wavefront holds
+__host__ __device__ inline int fast_strip_tiles(int N) { return 2 * ((N + 31) >> 5); }
+__host__ __device__ inline bool fast_strip_shape(int N, int K) {
+    const int nks = (K + 31) >> 5;
+    return N >= 2 && N <= kWaveCols && nks <= kFastSteps && fast_strip_tiles(N) * nks <= kFastBlocks;
+}
+
 // Kinds of scanned work-item counts.  Every kind except kPfxRows and kPfxSlow
 // counts aligned segments only (see below).
 enum PrefixKind {
@@ -51,7 +61,8 @@ struct PlanHeader {
     int32_t max_M, max_N, max_K;
     int32_t bad_segments;
     int32_t run_errors;      // bumped by kernels that refuse to run
-    int32_t pad_[31];
+    int32_t strip_rest;      // strip-class segments that do not fit the strip kernel's LDS window
+    int32_t pad_[30];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 

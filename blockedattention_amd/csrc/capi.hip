@@ -93,6 +93,7 @@ __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_pla
     info->max_M = h.max_M; info->max_N = h.max_N; info->max_K = h.max_K;
     info->bad_segments = h.bad_segments;
     info->run_errors = h.run_errors;
+    info->strip_rest = h.strip_rest;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 

@@ -432,6 +432,8 @@ __device__ __forceinline__ float exchange_row_stats(float (*sM)[16], float (*sL)
 // construction, no padding or swizzle to compute.  Segments whose B_g exceeds
 // the LDS window are walked in K slabs.
 constexpr int kLdsBlockBytes = 1024;
+constexpr int kSegWaves = 4;
+constexpr int kSegThreads = 64 * kSegWaves;
 // k-steps (of 32) whose A fragments a wavefront keeps in registers: 4 in the 128-register build, 2 in the
 // leaner build (larger K takes more slabs)
 template <int MAXNT> struct SlabSteps { static constexpr int value = MAXNT <= 8 ? 2 : 4; };
@@ -526,6 +528,241 @@ __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, c
     else strips_from_lds<DT, 16, FUSED, F32OUT, MAXNT>(s, a, lds, lds_blocks, r0, active, wave, nwaves);
 }
 
+
+// ------------------------------------------------------------ exact strips
+// The strip path for segments whose whole B_g fits the LDS window
+// (G * ceil(K/32) <= kFastBlocks blocks with G = the even tile count, K <= 128,
+// N >= 2): code specialised for the tile count, no per-tile conditions, B_g
+// copied to LDS once per workgroup and reused by every strip the workgroup takes.
+//
+// Layout.  The MFMA takes the strip's A rows as its first operand and B_g rows as
+// its second, so a lane holds four ROWS of one column slot.  Both operand orders
+// are free, and they are chosen so that memory order follows lane order:
+//   * column slot j of tile g is score column G*j + g, so lane j owns the G
+//     CONSECUTIVE columns [G*j, G*j + G) of each of its rows (register index = g);
+//   * operand row slot m is strip row 4*(m%4) + m/4, so register e of the lanes of
+//     row group rg (= lane/16) is strip row 4*e + rg: one store instruction (fixed
+//     e) covers the four consecutive strip rows 4e..4e+3, lane after lane, i.e. one
+//     contiguous run of 4*N elements of the output.
+// Adjacent lanes write adjacent addresses, which is what the memory pipeline
+// coalesces; a lane%16 = row layout writes 16 scattered pieces per instruction
+// and runs at a fraction of the store rate.
+// Ragged N: lanes j < J = N/G own full runs; if v = N - G*J > 0, lane J owns the
+// run [N-G, N) instead, overlapping lane J-1 in G-v columns (both lanes compute and
+// store identical values there); later lanes repeat column N-1 and store nothing.
+// Every store is a full run: there are no partial stores.  The row sum weights each
+// value by 1 or 0 (w[g]) so overlapped and repeated columns count once; the row
+// maximum needs no mask at all.
+
+typedef u32x4 __attribute__((aligned(2))) u32x4_unaligned;
+typedef uint32_t __attribute__((aligned(2))) u32_unaligned;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef f32x2 __attribute__((aligned(4))) f32x2_unaligned;
+
+__device__ __forceinline__ float min3(float a, float b, float c) {
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+// Reductions over the 16 lanes of a row group (lanes 16*rg .. 16*rg+15) with
+// data-parallel-primitive row rotations; every lane ends with the result.
+template <int CTRL> __device__ __forceinline__ float dpp_rot(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = __builtin_fmaxf(v, dpp_rot<0x128>(v));   // row_ror:8
+    v = __builtin_fmaxf(v, dpp_rot<0x124>(v));   // row_ror:4
+    v = __builtin_fmaxf(v, dpp_rot<0x122>(v));   // row_ror:2
+    v = __builtin_fmaxf(v, dpp_rot<0x121>(v));   // row_ror:1
+    return v;
+}
+__device__ __forceinline__ float row16_min(float v) {
+    v = __builtin_fminf(v, dpp_rot<0x128>(v));
+    v = __builtin_fminf(v, dpp_rot<0x124>(v));
+    v = __builtin_fminf(v, dpp_rot<0x122>(v));
+    v = __builtin_fminf(v, dpp_rot<0x121>(v));
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_rot<0x128>(v);
+    v += dpp_rot<0x124>(v);
+    v += dpp_rot<0x122>(v);
+    v += dpp_rot<0x121>(v);
+    return v;
+}
+
+// One row of a lane's run (G values scaled by factor) to memory as the widest stores.
+template <int DT, int G, bool F32OUT>
+__device__ __forceinline__ void store_run(char *dst, const f32x4 (&acc)[G], int e) {
+    if (!F32OUT) {
+        uint32_t w[G / 2];
+#pragma unroll
+        for (int k = 0; k < G / 2; ++k) w[k] = Elem<DT>::pack2(acc[2 * k][e], acc[2 * k + 1][e]);
+#pragma unroll
+        for (int k = 0; k + 4 <= G / 2; k += 4)
+            *reinterpret_cast<u32x4_unaligned *>(dst + 4 * k) = u32x4{w[k], w[k + 1], w[k + 2], w[k + 3]};
+        constexpr int kDone = (G / 2) & ~3;
+        if ((G / 2) & 2) *reinterpret_cast<u32x2_unaligned *>(dst + 4 * kDone) = u32x2{w[kDone], w[kDone + 1]};
+        if ((G / 2) & 1) *reinterpret_cast<u32_unaligned *>(dst + 4 * (G / 2 - 1)) = w[G / 2 - 1];
+    } else {
+#pragma unroll
+        for (int k = 0; k + 4 <= G; k += 4)
+            *reinterpret_cast<f32x4_unaligned *>(dst + 4 * k) =
+                f32x4{acc[k][e], acc[k + 1][e], acc[k + 2][e], acc[k + 3][e]};
+        if (G & 2) *reinterpret_cast<f32x2_unaligned *>(dst + 4 * (G - 2)) = f32x2{acc[G - 2][e], acc[G - 1][e]};
+    }
+}
+
+template <int DT, int G, bool FUSED, bool F32OUT>
+__device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, unsigned char *lds, int wave,
+                                             int first_strip, int strip_step) {
+    const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
+    const int K = s.K, N = s.N, M = s.M;
+    const int nks = (K + 31) >> 5;
+    const int strips = (M + kStripRows - 1) / kStripRows;
+    const SegRes res = make_res(s, a.A, a.B);
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+
+    // ---- this lane's run of columns
+    const int J = N / G, v = N - G * J;
+    const bool owner = j < J || (j == J && v > 0);
+    const int col0 = j < J ? G * j : N - G;                 // first column of the run (owners)
+
+    // ---- this wavefront's first A fragments: operand row slot j is strip row 4*(j%4) + j/4,
+    //      k-group rg; rows past M read as zeros (buffer range)
+    const int a_lane = ((4 * (j & 3) + (j >> 2)) * K + rg * 8) * 2;
+    u32x4 af[kFastSteps];
+    auto load_a = [&](int strip) {
+        const int voff = a_lane + strip * (kStripRows * 2) * K;
+#pragma unroll
+        for (int ks = 0; ks < kFastSteps; ++ks) {
+            af[ks] = zero;
+            if (ks < nks) af[ks] = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff + ks * 64, 0, 0);
+        }
+    };
+    load_a(first_strip);
+
+    // ---- B_g -> LDS, block (ks, g) at (ks * G + g) KiB, in MFMA operand order:
+    //      lane (slot j, k-group rg) brings 16 bytes of B_g row col0 + g
+    {
+        const uint16_t *bseg = (const uint16_t *)a.B + s.b;
+        const int brow0 = owner ? col0 : N - 1;
+        const int bstep = owner ? 1 : 0;
+        const int nblocks = nks * G;
+        for (int b = wave; b < nblocks; b += kSegWaves) {
+            const int ks = b / G, g = b - ks * G;
+            const int row = brow0 + bstep * g;
+            int kk = ks * 32 + rg * 8;
+            kk = kk < K ? kk : 0;            // ragged last k-step: valid data, multiplied by a zero A fragment
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bseg + row * K + kk),
+                                             (__attribute__((address_space(3))) void *)(lds + b * kLdsBlockBytes),
+                                             16, 0, 0);
+        }
+    }
+    // weights of the row sum: 1 for columns this lane alone accounts for
+    float w[G];
+    if (FUSED) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) w[g] = (j < J || (j == J && g >= G - v)) ? 1.f : 0.f;
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    const unsigned char *blk = lds + lane * 16;
+    const bool ragged_k = (K & 31) != 0;
+    const bool k_live = (nks - 1) * 32 + rg * 8 < K;
+    const float c = a.scale * kLog2e;
+    constexpr int kOutBytes = F32OUT ? 4 : 2;
+    char *const obase = reinterpret_cast<char *>(a.out) + s.o * kOutBytes;
+    const uint32_t run_off = (uint32_t)(rg * N + col0) * kOutBytes;
+
+    for (int strip = first_strip; strip < strips; strip += strip_step) {
+        if (ragged_k) {
+#pragma unroll
+            for (int ks = 0; ks < kFastSteps; ++ks)
+                if (ks == nks - 1) af[ks] = k_live ? af[ks] : zero;
+        }
+        f32x4 acc[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + g * kLdsBlockBytes);
+            acc[g] = Elem<DT>::mfma(af[0], bf, f32x4{0.f, 0.f, 0.f, 0.f});
+        }
+#pragma unroll
+        for (int ks = 1; ks < kFastSteps; ++ks) {
+            if (ks < nks) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + (ks * G + g) * kLdsBlockBytes);
+                    acc[g] = Elem<DT>::mfma(af[ks], bf, acc[g]);
+                }
+            }
+        }
+        load_a(strip + strip_step);          // next strip's fragments fly under the softmax and the stores
+
+        if (FUSED) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float ext;
+                if (c >= 0.f) {
+                    ext = acc[0][e];
+#pragma unroll
+                    for (int g = 1; g + 1 < G; g += 2) ext = max3(ext, acc[g][e], acc[g + 1][e]);
+                    ext = row16_max(__builtin_fmaxf(ext, acc[G - 1][e]));
+                } else {
+                    ext = acc[0][e];
+#pragma unroll
+                    for (int g = 1; g + 1 < G; g += 2) ext = min3(ext, acc[g][e], acc[g + 1][e]);
+                    ext = row16_min(__builtin_fminf(ext, acc[G - 1][e]));
+                }
+                const float bias = -((__builtin_fabsf(ext) == INFINITY) ? 0.f : ext) * c;
+                float sum = 0.f;
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const float pr = __builtin_amdgcn_exp2f(fmaf(acc[g][e], c, bias));
+                    acc[g][e] = pr;
+                    sum = fmaf(pr, w[g], sum);
+                }
+                const float inv = __builtin_amdgcn_rcpf(row16_sum(sum));
+#pragma unroll
+                for (int g = 0; g < G; ++g) acc[g][e] *= inv;
+            }
+        }
+
+        if (owner) {
+            const int r0 = strip * kStripRows;
+            char *dst = obase + (size_t)r0 * N * kOutBytes + run_off;
+            const int row_stride4 = 4 * N * kOutBytes;
+            if (r0 + kStripRows <= M) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) store_run<DT, G, F32OUT>(dst + e * row_stride4, acc, e);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (r0 + 4 * e + rg < M) store_run<DT, G, F32OUT>(dst + e * row_stride4, acc, e);
+            }
+        }
+    }
+}
+
+template <int DT, bool FUSED, bool F32OUT, int MAXNT>
+__device__ __forceinline__ void strips_exact_dispatch(int tiles, const Seg &s, const RunArgs &a, unsigned char *lds,
+                                                      int wave, int first_strip, int strip_step) {
+#define BA_EXACT(G_) case G_: strips_exact<DT, G_, FUSED, F32OUT>(s, a, lds, wave, first_strip, strip_step); break;
+    switch (tiles) {
+        BA_EXACT(2) BA_EXACT(4) BA_EXACT(6) BA_EXACT(8)
+        default:
+            if (MAXNT > 8) {
+                switch (tiles) {
+                    BA_EXACT(10) BA_EXACT(12) BA_EXACT(14) BA_EXACT(16)
+                    default: break;
+                }
+            }
+            break;
+    }
+#undef BA_EXACT
+}
+
 // ------------------------------------------------------------------ kernels
 // segment_kernel   grid (segment, head, z): one workgroup per segment and head;
 //                  its wavefronts take the segment's 16-row strips (N <= 256),
@@ -536,8 +773,6 @@ __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, c
 // split_kernel / wide_kernel  fused, N > 256: one 16-wave workgroup per strip.
 // The list kernels loop `for (item = first; item < total; item += stride)` with
 // the total read from the plan, so any grid size is correct.
-constexpr int kSegWaves = 4;
-constexpr int kSegThreads = 64 * kSegWaves;
 
 // The header fields every kernel checks, fetched as one batch of scalar loads
 // (no branch between them).  The segment count comes with the launch, so the
@@ -569,7 +804,10 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
     const bool ok = header_ok(a);
     const Seg s = load_seg(pv, g, h, a);
     const int kind = pv.recs[g].kind;
-    if (!ok) { report_mismatch(a); return; }
+    if (!ok) {
+        if (!(a.flags & kFlagFastStrips)) report_mismatch(a);   // else the strip kernel of this call has reported
+        return;
+    }
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int first = blockIdx.z * kSegWaves + wave, stride = gridDim.z * kSegWaves;
     const bool mfma_ok = (a.flags & kFlagMfmaOk) != 0;
@@ -581,6 +819,7 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
         return;
     }
     if (kind == kSegStrip) {
+        if ((a.flags & kFlagFastStrips) && fast_strip_shape(s.N, s.K) && fast_strip_tiles(s.N) <= MAXNT) return;
         // One strip per wavefront; blockIdx.z selects the group of kSegWaves strips.
         const int strips = (s.M + kStripRows - 1) / kStripRows;
         const int nt = (s.N + 15) >> 4;
@@ -593,6 +832,28 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
     } else if (kind == kSegPackLead) {
         if (first == 0) wave_pack<DT, FUSED, F32OUT>(pv, g, pv.recs[g].packLen, h, a);
     }
+}
+
+// strip_kernel: the strip-class segments whose B_g fits the LDS window, nothing else.
+// Grid (segment, head, z); the workgroups with the same (segment, head) share the
+// segment's strips round-robin.
+template <int DT, bool FUSED, bool F32OUT, int MAXNT>
+__global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(RunArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    const int g = blockIdx.x;
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
+    const int64_t h = blockIdx.y;
+    const bool ok = header_ok(a);
+    const Seg s = load_seg(pv, g, h, a);
+    const int kind = pv.recs[g].kind;
+    if (!ok) { report_mismatch(a); return; }
+    if (kind != kSegStrip) return;
+    const int tiles = fast_strip_tiles(s.N);
+    if (!fast_strip_shape(s.N, s.K) | (tiles > MAXNT)) return;
+    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int first = blockIdx.z * kSegWaves + wave, step = gridDim.z * kSegWaves;
+    if ((int)blockIdx.z * kSegWaves * kStripRows >= s.M) return;   // no strip for this workgroup
+    strips_exact_dispatch<DT, FUSED, F32OUT, MAXNT>(tiles, s, a, lds, wave, first, step);
 }
 
 template <int DT>
@@ -751,9 +1012,36 @@ static int launch_set(const RunArgs &args, int64_t nseg, const ba_plan_info *inf
         g_split = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, info->split_items) : 0;
         g_wide = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, info->wide_items) : 0;
     }
+    // Strip kernel: with a plan summary, launched when strip-class segments exist; it takes those whose
+    // B_g fits its window, the segment kernel below takes the rest (and is skipped when nothing is left).
+    RunArgs args_rest = args;
+    if (nseg > 0 && mfma_ok && (!info || info->strip_items > 0)) {
+        int64_t blocks = kFastBlocks, zf = 2;
+        bool lean = false;
+        if (info) {
+            const int64_t nt = fast_strip_tiles((int)std::min<int64_t>(std::max<int64_t>(info->max_N, 1), kWaveCols));
+            const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
+            blocks = std::min<int64_t>(kFastBlocks, nt * nks);
+            lean = info->max_N <= 128;
+            // enough workgroups to fill the machine, at most one per kSegWaves strips
+            const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(info->max_M, 1), kStripRows), kSegWaves);
+            const int64_t want = ceil_div((int64_t)cus * 8, std::max<int64_t>(1, nseg * (int64_t)H));
+            zf = std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
+        }
+        RunArgs fa = args;
+        fa.lds_blocks = (int)blocks;
+        const dim3 grid((unsigned)nseg, H, (unsigned)zf);
+        const size_t lds_bytes = (size_t)blocks * kLdsBlockBytes;
+        if (lean)
+            hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
+        else
+            hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
+        args_rest.flags |= kFlagFastStrips;
+        if (info && info->strip_rest == 0 && info->pack_items + info->slow_items == 0) seg_work = false;
+    }
     if (nseg > 0 && seg_work) {
         // LDS window for B_g: whole B_g of the largest strip-class segment if known, else 32 KiB.
-        RunArgs seg_args = args;
+        RunArgs seg_args = args_rest;
         int64_t blocks = 32;
         if (info) {
             const int64_t nt = ceil_div(std::min<int64_t>(std::max<int64_t>(info->max_N, 1), kWaveCols), 16);

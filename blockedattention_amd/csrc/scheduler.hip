@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
     __shared__ __attribute__((aligned(16))) int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads];
     __shared__ int32_t sPack[kSchedThreads];
-    __shared__ int32_t sRed[kSchedWaves][4];
+    __shared__ int32_t sRed[kSchedWaves][5];
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6), lane = lane_id();
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
 
     int64_t base64[3] = {0, 0, 0};
     int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0};
-    int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
+    int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0, nrest = 0;
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
 
     for (int64_t chunk = 0; chunk < nseg || chunk == 0; chunk += kSchedThreads) {
@@ -220,6 +220,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             }
         }
         maxM = max(maxM, mi); maxN = max(maxN, ni); maxK = max(maxK, ki); nbad += bad ? 1 : 0;
+        nrest += (a.kind == 0 && mfma_ok && strips > 0 && ni <= kWaveCols && !fast_strip_shape(ni, ki)) ? 1 : 0;
 #pragma unroll
         for (int q = 0; q < kNumPrefix; ++q) base32[q] += t32[q];
         if (!offsets_given) {
@@ -234,7 +235,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     // wavefront, then thread 0 folds the 16 partial results.
     maxM = wave_max_nonneg(maxM); maxN = wave_max_nonneg(maxN); maxK = wave_max_nonneg(maxK);
     nbad = __builtin_amdgcn_readlane(wave_inclusive_scan(nbad), 63);
-    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; }
+    nrest = __builtin_amdgcn_readlane(wave_inclusive_scan(nrest), 63);
+    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; sRed[wave][4] = nrest; }
     __syncthreads();
 
     if (tid == 0) {
@@ -249,9 +251,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             if (a.a2) a.a2[nseg] = D2;
             if (a.aO) a.aO[nseg] = DO;
         }
-        int32_t rM = 0, rN = 0, rK = 0, rBad = 0;
+        int32_t rM = 0, rN = 0, rK = 0, rBad = 0, rRest = 0;
         for (int w = 0; w < kSchedWaves; ++w) {
-            rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3];
+            rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3]; rRest += sRed[w][4];
         }
         for (int q = 0; q < kNumPrefix; ++q) pv.pfx[q][nseg] = base32[q];
         PlanHeader *h = pv.hdr;
@@ -265,6 +267,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->max_M = rM; h->max_N = rN; h->max_K = rK;
         h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
         h->run_errors = 0;
+        h->strip_rest = rRest;
     }
 }
 

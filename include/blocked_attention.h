@@ -65,7 +65,7 @@ typedef struct ba_plan_info {
     int32_t max_M, max_N, max_K;
     int32_t bad_segments;   /* segments rejected by the device-side checks */
     int32_t run_errors;     /* kernels that refused to run against this plan */
-    int32_t reserved;
+    int32_t strip_rest;     /* strip-class segments too large for the strip kernel's LDS window */
 } ba_plan_info;
 
 const char *ba_status_string(int status);
