@@ -28,7 +28,7 @@ constexpr int kFastSteps = 4;     // k-steps of 32 whose A fragments a wavefront
 __host__ __device__ inline int fast_strip_tiles(int N) { return 2 * ((N + 31) >> 5); }
 __host__ __device__ inline bool fast_strip_shape(int N, int K) {
     const int nks = (K + 31) >> 5;
-    return N >= 2 && N <= kWaveCols && nks <= kFastSteps && fast_strip_tiles(N) * nks <= kFastBlocks;
+    return N >= 2 && N <= kWaveCols && nks >= 1 && nks <= kFastSteps && fast_strip_tiles(N) * nks <= kFastBlocks;
 }
 
 // Kinds of scanned work-item counts.  Every kind except kPfxRows and kPfxSlow

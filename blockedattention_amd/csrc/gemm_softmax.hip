@@ -559,37 +559,23 @@ typedef uint32_t __attribute__((aligned(2))) u32_unaligned;
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef f32x2 __attribute__((aligned(4))) f32x2_unaligned;
 
-__device__ __forceinline__ float min3(float a, float b, float c) {
-    float r;
-    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
 // Reductions over the 16 lanes of a row group (lanes 16*rg .. 16*rg+15) with
-// data-parallel-primitive row rotations; every lane ends with the result.
-template <int CTRL> __device__ __forceinline__ float dpp_rot(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float row16_max(float v) {
-    v = __builtin_fmaxf(v, dpp_rot<0x128>(v));   // row_ror:8
-    v = __builtin_fmaxf(v, dpp_rot<0x124>(v));   // row_ror:4
-    v = __builtin_fmaxf(v, dpp_rot<0x122>(v));   // row_ror:2
-    v = __builtin_fmaxf(v, dpp_rot<0x121>(v));   // row_ror:1
-    return v;
-}
-__device__ __forceinline__ float row16_min(float v) {
-    v = __builtin_fminf(v, dpp_rot<0x128>(v));
-    v = __builtin_fminf(v, dpp_rot<0x124>(v));
-    v = __builtin_fminf(v, dpp_rot<0x122>(v));
-    v = __builtin_fminf(v, dpp_rot<0x121>(v));
-    return v;
-}
-__device__ __forceinline__ float row16_sum(float v) {
-    v += dpp_rot<0x128>(v);
-    v += dpp_rot<0x124>(v);
-    v += dpp_rot<0x122>(v);
-    v += dpp_rot<0x121>(v);
-    return v;
-}
+// data-parallel-primitive row rotations: x = op(rotate(x), x) for rotations by 8,
+// 4, 2, 1, after which every lane holds the result.  Four independent values go
+// through the steps side by side, which also keeps a rotation three instructions
+// away from the write of its source (the hardware needs two).
+#define BA_ROT_STEP(OP, ROT)                                                   \
+    OP " %0, %0, %0 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
+    OP " %1, %1, %1 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
+    OP " %2, %2, %2 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
+    OP " %3, %3, %3 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"
+#define BA_ROT_REDUCE(OP)                                                                      \
+    asm("s_nop 1\n" BA_ROT_STEP(OP, 8) BA_ROT_STEP(OP, 4) BA_ROT_STEP(OP, 2) BA_ROT_STEP(OP, 1) \
+        : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]))
+__device__ __forceinline__ void row16_max4(float (&x)[4]) { BA_ROT_REDUCE("v_max_f32_dpp"); }
+__device__ __forceinline__ void row16_sum4(float (&x)[4]) { BA_ROT_REDUCE("v_add_f32_dpp"); }
+#undef BA_ROT_REDUCE
+#undef BA_ROT_STEP
 
 // One row of a lane's run (G values scaled by factor) to memory as the widest stores.
 template <int DT, int G, bool F32OUT>
@@ -635,10 +621,8 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
     auto load_a = [&](int strip) {
         const int voff = a_lane + strip * (kStripRows * 2) * K;
 #pragma unroll
-        for (int ks = 0; ks < kFastSteps; ++ks) {
-            af[ks] = zero;
+        for (int ks = 0; ks < kFastSteps; ++ks)
             if (ks < nks) af[ks] = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff + ks * 64, 0, 0);
-        }
     };
     load_a(first_strip);
 
@@ -671,7 +655,11 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
     const unsigned char *blk = lds + lane * 16;
     const bool ragged_k = (K & 31) != 0;
     const bool k_live = (nks - 1) * 32 + rg * 8 < K;
-    const float c = a.scale * kLog2e;
+    // A negative softmax scale is applied as |scale| to negated scores: the sign bits of the A
+    // fragments are flipped, so the row maximum below is always the value to subtract.
+    const float c_signed = a.scale * kLog2e;
+    const bool negate = FUSED && c_signed < 0.f;
+    const float c = __builtin_fabsf(c_signed);
     constexpr int kOutBytes = F32OUT ? 4 : 2;
     char *const obase = reinterpret_cast<char *>(a.out) + s.o * kOutBytes;
     const uint32_t run_off = (uint32_t)(rg * N + col0) * kOutBytes;
@@ -681,6 +669,11 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
 #pragma unroll
             for (int ks = 0; ks < kFastSteps; ++ks)
                 if (ks == nks - 1) af[ks] = k_live ? af[ks] : zero;
+        }
+        if (negate) {
+#pragma unroll
+            for (int ks = 0; ks < kFastSteps; ++ks)
+                if (ks < nks) af[ks] ^= u32x4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
         }
         f32x4 acc[G];
 #pragma unroll
@@ -701,29 +694,30 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         load_a(strip + strip_step);          // next strip's fragments fly under the softmax and the stores
 
         if (FUSED) {
+            float ext[4], sum[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                float ext;
-                if (c >= 0.f) {
-                    ext = acc[0][e];
+                ext[e] = acc[0][e];
 #pragma unroll
-                    for (int g = 1; g + 1 < G; g += 2) ext = max3(ext, acc[g][e], acc[g + 1][e]);
-                    ext = row16_max(__builtin_fmaxf(ext, acc[G - 1][e]));
-                } else {
-                    ext = acc[0][e];
+                for (int g = 1; g + 1 < G; g += 2) ext[e] = max3(ext[e], acc[g][e], acc[g + 1][e]);
+                ext[e] = max3(ext[e], acc[G - 1][e], acc[G - 1][e]);
+            }
+            row16_max4(ext);
 #pragma unroll
-                    for (int g = 1; g + 1 < G; g += 2) ext = min3(ext, acc[g][e], acc[g + 1][e]);
-                    ext = row16_min(__builtin_fminf(ext, acc[G - 1][e]));
-                }
-                const float bias = -((__builtin_fabsf(ext) == INFINITY) ? 0.f : ext) * c;
-                float sum = 0.f;
+            for (int e = 0; e < 4; ++e) {
+                const float bias = -((__builtin_fabsf(ext[e]) == INFINITY) ? 0.f : ext[e]) * c;
+                sum[e] = 0.f;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     const float pr = __builtin_amdgcn_exp2f(fmaf(acc[g][e], c, bias));
                     acc[g][e] = pr;
-                    sum = fmaf(pr, w[g], sum);
+                    sum[e] = fmaf(pr, w[g], sum[e]);
                 }
-                const float inv = __builtin_amdgcn_rcpf(row16_sum(sum));
+            }
+            row16_sum4(sum);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float inv = __builtin_amdgcn_rcpf(sum[e]);
 #pragma unroll
                 for (int g = 0; g < G; ++g) acc[g][e] *= inv;
             }
