@@ -1,0 +1,90 @@
+// Device code shared by the MFMA kernels (strip, segment and tile kernels):
+// segment views, buffer descriptors, plan checks, cross-lane reductions.
+#pragma once
+#include "ba_device.hpp"
+#include "ba_host.hpp"
+
+namespace ba {
+
+struct Seg {
+    int M, N, K;
+    int64_t a, b, o;  // element offsets of the segment inside A, B, out (head included)
+};
+
+// Buffer resources of one segment.  Operand loads go through a raw buffer
+// descriptor whose range is exactly the segment: the address is one 32-bit lane
+// offset plus a scalar offset, and anything past the segment's end (rows >= M
+// of a ragged strip, columns >= N of a ragged tile) reads as zero instead of
+// being clamped in code.
+struct SegRes {
+    __amdgpu_buffer_rsrc_t a, b;
+};
+
+constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
+
+__device__ __forceinline__ SegRes make_res(const Seg &s, const void *A, const void *B) {
+    SegRes r;
+    r.a = __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)A + s.a), 0, s.M * s.K * 2, kRsrcFlags);
+    r.b = __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)B + s.b), 0, s.N * s.K * 2, kRsrcFlags);
+    return r;
+}
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;   // one instruction for two new elements; fmaxf() would add a canonicalising max per operand
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+
+typedef u32x2 __attribute__((aligned(2))) u32x2_unaligned;
+typedef f32x4 __attribute__((aligned(4))) f32x4_unaligned;
+typedef u32x4 __attribute__((aligned(2))) u32x4_unaligned;
+typedef uint32_t __attribute__((aligned(2))) u32_unaligned;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef f32x2 __attribute__((aligned(4))) f32x2_unaligned;
+
+// Reductions over the 16 lanes of a row group (lanes 16*rg .. 16*rg+15) with
+// data-parallel-primitive row rotations: x = op(rotate(x), x) for rotations by 8,
+// 4, 2, 1, after which every lane holds the result.  Four independent values go
+// through the steps side by side, which also keeps a rotation three instructions
+// away from the write of its source (the hardware needs two).
+#define BA_ROT_STEP(OP, ROT)                                                   \
+    OP " %0, %0, %0 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
+    OP " %1, %1, %1 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
+    OP " %2, %2, %2 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
+    OP " %3, %3, %3 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"
+#define BA_ROT_REDUCE(OP)                                                                      \
+    asm("s_nop 1\n" BA_ROT_STEP(OP, 8) BA_ROT_STEP(OP, 4) BA_ROT_STEP(OP, 2) BA_ROT_STEP(OP, 1) \
+        : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]))
+__device__ __forceinline__ void row16_max4(float (&x)[4]) { BA_ROT_REDUCE("v_max_f32_dpp"); }
+__device__ __forceinline__ void row16_sum4(float (&x)[4]) { BA_ROT_REDUCE("v_add_f32_dpp"); }
+#undef BA_ROT_REDUCE
+#undef BA_ROT_STEP
+
+__device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
+    const SegRec r = load_rec(pv.recs, g);   // scalar loads
+    Seg s;
+    s.M = r.M; s.N = r.N; s.K = r.K;
+    s.a = h * a.Dm1 + r.off1;
+    s.b = h * a.Dm2 + r.off2;
+    s.o = h * a.Dout + r.offO;
+    return s;
+}
+
+// The header fields every kernel checks, fetched as one batch of scalar loads
+// (no branch between them).  The segment count comes with the launch, so the
+// addresses of the plan's arrays do not wait for the header either.
+__device__ __forceinline__ bool header_ok(const RunArgs &a) {
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+    const uint32_t magic = hdr->magic;
+    const int nseg = hdr->nseg, kind = hdr->kind, bad = hdr->bad_segments;
+    const int64_t d1 = hdr->Dm1, d2 = hdr->Dm2, dO = hdr->Dout;
+    return (magic == kPlanMagic) & (nseg == a.nseg) & (kind == 0) & (bad == 0) & (d1 == a.Dm1) & (d2 == a.Dm2) &
+           (dO == a.Dout);
+}
+__device__ __forceinline__ void report_mismatch(const RunArgs &a) {
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+        atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+}
+
+}  // namespace ba

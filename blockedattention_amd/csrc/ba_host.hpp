@@ -13,7 +13,9 @@ enum RunFlags : int {
     kFlagTranspose2 = 2,   // B segments stored K x N
     kFlagMfmaOk = 4,       // layouts, base pointers and head strides allow 16-byte operand loads
     kFlagOutF32 = 8,       // fused path writes fp32 probabilities
-    kFlagFastStrips = 16   // the strip kernel runs in the same call and takes the segments that fit its window
+    kFlagFastStrips = 16,  // the strip kernel runs in the same call and takes the segments that fit its window
+    kFlagTiles = 32,       // the tile kernel runs in the same call and takes the large segments
+    kFlagQuiet = 64        // an earlier launch of the same call reports a plan that does not match
 };
 
 struct RunArgs {
@@ -35,6 +37,9 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
 // info: optional host copy of the plan summary (from ba_plan_read), or nullptr.
 int launch_strips(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
                   hipStream_t stream);
+// The tile kernel over the large segments (see tile_segment()).
+int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
+                 hipStream_t stream);
 int launch_gemm_f32(const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,
                    float scale, const ba_plan_info *info, hipStream_t stream);

@@ -79,6 +79,14 @@ enum SegKind : int32_t {
     kSegSlow = 6         // not 16-byte aligned (K % 8, odd offsets) or too large for 32-bit offsets
 };
 
+// Segments the tile kernel takes: N > 256, or strip-class segments too large for the strip
+// kernel's LDS window that have at least one full chunk of columns.
+constexpr int kTileCols = 64;
+__host__ __device__ inline bool tile_segment(int kind, int N, int K) {
+    if (kind == kSegSplit || kind == kSegWide) return true;
+    return kind == kSegStrip && !fast_strip_shape(N, K) && N >= kTileCols;
+}
+
 // Everything a kernel needs to know about one segment, in one aligned record
 // (three 16-byte scalar loads).
 struct alignas(16) SegRec {

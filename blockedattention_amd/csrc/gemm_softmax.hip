@@ -21,36 +21,12 @@
 // take an element-wise loader into the same MFMA code.
 #include <algorithm>
 
-#include "ba_device.hpp"
-#include "ba_host.hpp"
+#include "ba_gemm_common.hpp"
 
 namespace ba {
 
 constexpr int kGroupThreads = 64 * kWavesPerGroup;
 constexpr int kMaxTiles = kWaveCols / 16;  // 16 MFMA tiles per wavefront
-
-struct Seg {
-    int M, N, K;
-    int64_t a, b, o;  // element offsets of the segment inside A, B, out (head included)
-};
-
-// Buffer resources of one segment.  Operand loads go through a raw buffer
-// descriptor whose range is exactly the segment: the address is one 32-bit lane
-// offset plus a scalar offset, and anything past the segment's end (rows >= M
-// of a ragged strip, columns >= N of a ragged tile) reads as zero instead of
-// being clamped in code.
-struct SegRes {
-    __amdgpu_buffer_rsrc_t a, b;
-};
-
-constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
-
-__device__ __forceinline__ SegRes make_res(const Seg &s, const void *A, const void *B) {
-    SegRes r;
-    r.a = __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)A + s.a), 0, s.M * s.K * 2, kRsrcFlags);
-    r.b = __builtin_amdgcn_make_buffer_rsrc((void *)((const uint16_t *)B + s.b), 0, s.N * s.K * 2, kRsrcFlags);
-    return r;
-}
 
 // ------------------------------------------------------------ operand loads
 __device__ __forceinline__ u32x4 load_frag_fast(const uint16_t *__restrict__ row_ptr, int kk, int K) {
@@ -163,12 +139,6 @@ __device__ __forceinline__ void stage_scores(f32x4 (&acc)[kMaxTiles], const Seg 
 }
 
 // ------------------------------------------------------------ local softmax
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    float r;   // one instruction for two new elements; fmaxf() would add a canonicalising max per operand
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
-
 // Brings raw scores into the form the softmax below takes: the multiplier c =
 // scale * log2(e) made non-negative (scores negated for a negative scale, set
 // to zero for a zero scale, where every probability is 1/N), and the columns of
@@ -237,8 +207,6 @@ __device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int nt, f
 // or 16-byte (fp32 output) store whatever the address: row starts are only
 // element-aligned (odd N), and the memory pipeline takes vector stores at any
 // element alignment.  Only the ragged last tile of a row uses element stores.
-typedef u32x2 __attribute__((aligned(2))) u32x2_unaligned;
-typedef f32x4 __attribute__((aligned(4))) f32x4_unaligned;
 
 template <int DT, bool F32OUT>
 __device__ __forceinline__ void store_quad(void *__restrict__ out, int64_t e, const f32x4 &v, int valid) {
@@ -307,16 +275,6 @@ __device__ __forceinline__ void wave_strip_dispatch(int nt, const Seg &s, const 
     else if (nt <= 4) wave_strip<DT, 4, FUSED, F32OUT>(nt, s, a, r0, c0);
     else if (nt <= 8) wave_strip<DT, 8, FUSED, F32OUT>(nt, s, a, r0, c0);
     else wave_strip<DT, 16, FUSED, F32OUT>(nt, s, a, r0, c0);
-}
-
-__device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
-    const SegRec r = load_rec(pv.recs, g);   // scalar loads
-    Seg s;
-    s.M = r.M; s.N = r.N; s.K = r.K;
-    s.a = h * a.Dm1 + r.off1;
-    s.b = h * a.Dm2 + r.off2;
-    s.o = h * a.Dout + r.offO;
-    return s;
 }
 
 template <int DT, bool FUSED>
@@ -554,29 +512,6 @@ __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, c
 // value by 1 or 0 (w[g]) so overlapped and repeated columns count once; the row
 // maximum needs no mask at all.
 
-typedef u32x4 __attribute__((aligned(2))) u32x4_unaligned;
-typedef uint32_t __attribute__((aligned(2))) u32_unaligned;
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef f32x2 __attribute__((aligned(4))) f32x2_unaligned;
-
-// Reductions over the 16 lanes of a row group (lanes 16*rg .. 16*rg+15) with
-// data-parallel-primitive row rotations: x = op(rotate(x), x) for rotations by 8,
-// 4, 2, 1, after which every lane holds the result.  Four independent values go
-// through the steps side by side, which also keeps a rotation three instructions
-// away from the write of its source (the hardware needs two).
-#define BA_ROT_STEP(OP, ROT)                                                   \
-    OP " %0, %0, %0 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
-    OP " %1, %1, %1 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
-    OP " %2, %2, %2 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"            \
-    OP " %3, %3, %3 row_ror:" #ROT " row_mask:0xf bank_mask:0xf\n"
-#define BA_ROT_REDUCE(OP)                                                                      \
-    asm("s_nop 1\n" BA_ROT_STEP(OP, 8) BA_ROT_STEP(OP, 4) BA_ROT_STEP(OP, 2) BA_ROT_STEP(OP, 1) \
-        : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]))
-__device__ __forceinline__ void row16_max4(float (&x)[4]) { BA_ROT_REDUCE("v_max_f32_dpp"); }
-__device__ __forceinline__ void row16_sum4(float (&x)[4]) { BA_ROT_REDUCE("v_add_f32_dpp"); }
-#undef BA_ROT_REDUCE
-#undef BA_ROT_STEP
-
 // One row of a lane's run (G values scaled by factor) to memory as the widest stores.
 template <int DT, int G, bool F32OUT>
 __device__ __forceinline__ void store_run(char *dst, const f32x4 (&acc)[G], int e) {
@@ -768,22 +703,6 @@ __device__ __forceinline__ void strips_exact_dispatch(int tiles, const Seg &s, c
 // The list kernels loop `for (item = first; item < total; item += stride)` with
 // the total read from the plan, so any grid size is correct.
 
-// The header fields every kernel checks, fetched as one batch of scalar loads
-// (no branch between them).  The segment count comes with the launch, so the
-// addresses of the plan's arrays do not wait for the header either.
-__device__ __forceinline__ bool header_ok(const RunArgs &a) {
-    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const uint32_t magic = hdr->magic;
-    const int nseg = hdr->nseg, kind = hdr->kind, bad = hdr->bad_segments;
-    const int64_t d1 = hdr->Dm1, d2 = hdr->Dm2, dO = hdr->Dout;
-    return (magic == kPlanMagic) & (nseg == a.nseg) & (kind == 0) & (bad == 0) & (d1 == a.Dm1) & (d2 == a.Dm2) &
-           (dO == a.Dout);
-}
-__device__ __forceinline__ void report_mismatch(const RunArgs &a) {
-    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
-        atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
-}
-
 // MAXNT = 8 is the build for batches whose widest segment has N <= 128: half the
 // accumulator registers, half again as many resident wavefronts.  The host picks it from
 // the plan summary; without a summary the 16-tile build runs.
@@ -799,13 +718,14 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
     const Seg s = load_seg(pv, g, h, a);
     const int kind = pv.recs[g].kind;
     if (!ok) {
-        if (!(a.flags & kFlagFastStrips)) report_mismatch(a);   // else the strip kernel of this call has reported
+        if (!(a.flags & kFlagQuiet)) report_mismatch(a);
         return;
     }
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int first = blockIdx.z * kSegWaves + wave, stride = gridDim.z * kSegWaves;
     const bool mfma_ok = (a.flags & kFlagMfmaOk) != 0;
     if (kind == kSegEmpty) return;
+    if (mfma_ok && (a.flags & kFlagTiles) && tile_segment(kind, s.N, s.K)) return;
     if (!mfma_ok || kind == kSegSlow) {
         // Element-wise path.  With MFMA ruled out for the whole launch this also
         // covers the segments the list kernels would have taken.
@@ -840,7 +760,10 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
     const bool ok = header_ok(a);
     const Seg s = load_seg(pv, g, h, a);
     const int kind = pv.recs[g].kind;
-    if (!ok) { report_mismatch(a); return; }
+    if (!ok) {
+        if (!(a.flags & kFlagQuiet)) report_mismatch(a);
+        return;
+    }
     if (kind != kSegStrip) return;
     const int tiles = fast_strip_tiles(s.N);
     if (!fast_strip_shape(s.N, s.K) | (tiles > MAXNT)) return;
@@ -850,166 +773,38 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
     strips_exact_dispatch<DT, FUSED, F32OUT, MAXNT>(tiles, s, a, lds, wave, first, step);
 }
 
-template <int DT>
-__global__ __launch_bounds__(kSegThreads, 4) void gemm_large_kernel(RunArgs a) {
-    if (!header_ok(a) | !(a.flags & kFlagMfmaOk)) return;     // the segment kernel reports and covers these cases
-    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const PlanRO pv = plan_ro(a.plan, a.nseg);
-    const int wave = uniform((int)(threadIdx.x >> 6));
-    const int per_head = (int)hdr->totals[kPfxGemm];
-    const ConstI32 pfx = pv.pfx[kPfxGemm];
-    const int64_t h = blockIdx.y;
-    for (int i = blockIdx.x * kSegWaves + wave; i < per_head; i += gridDim.x * kSegWaves) {
-        const int g = prefix_search(pfx, a.nseg, i);
-        const int local = i - pfx[g];
-        const Seg s = load_seg(pv, g, h, a);
-        const int chunks = (s.N + kWaveCols - 1) / kWaveCols;
-        const int r0 = (local / chunks) * kStripRows, c0 = (local % chunks) * kWaveCols;
-        const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
-        wave_strip_dispatch<DT, false, false>(nt, s, a, r0, c0);
-    }
-}
-
-// 256 < N <= 4096: each wavefront of the workgroup owns 256 columns of the strip.
-template <int DT, bool F32OUT>
-__global__ __launch_bounds__(kGroupThreads) void split_kernel(RunArgs a) {
-    // Two copies: consecutive strips alternate, so a wavefront that runs ahead
-    // never overwrites statistics its neighbours are still reading.
-    __shared__ float sM[2][kWavesPerGroup][16];
-    __shared__ float sL[2][kWavesPerGroup][16];
-    if (!header_ok(a) | !(a.flags & kFlagMfmaOk)) return;
-    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const PlanRO pv = plan_ro(a.plan, a.nseg);
-    const int wave = uniform((int)(threadIdx.x >> 6));
-    const int per_head = (int)hdr->totals[kPfxSplit];
-    const ConstI32 pfx = pv.pfx[kPfxSplit];
-    const int64_t h = blockIdx.y;
-    const float c_raw = a.scale * kLog2e;
-    const float c = c_raw < 0.f ? -c_raw : (c_raw == 0.f ? 1.f : c_raw);   // what prepare_scores leaves
-    int xchg = 0;
-    for (int i = blockIdx.x; i < per_head; i += gridDim.x) {
-        const int g = prefix_search(pfx, a.nseg, i);
-        const int r0 = (i - pfx[g]) * kStripRows;
-        const Seg s = load_seg(pv, g, h, a);
-        const SegRes res = make_res(s, a.A, a.B);
-        const int c0 = wave * kWaveCols;
-        const int nt = max(0, min(kMaxTiles, (s.N - c0 + 15) >> 4));
-        f32x4 acc[kMaxTiles];
-        float m = -INFINITY, l = 0.f;
-#define BA_SPLIT_STAGE(NT)                              \
-    {                                                   \
-        float cc = c_raw;                               \
-        stage_scores<DT, NT>(acc, s, res, r0, c0);      \
-        prepare_scores<NT>(acc, nt, s.N, c0, cc);       \
-        local_softmax<NT>(acc, nt, cc, m, l);           \
-    }
-        if (nt > 8) BA_SPLIT_STAGE(16)
-        else if (nt > 4) BA_SPLIT_STAGE(8)
-        else if (nt > 2) BA_SPLIT_STAGE(4)
-        else if (nt > 1) BA_SPLIT_STAGE(2)
-        else if (nt > 0) BA_SPLIT_STAGE(1)
-#undef BA_SPLIT_STAGE
-        const int buf = xchg & 1;
-        ++xchg;
-        float gshift, ginv;
-        const float factor = exchange_row_stats(sM[buf], sL[buf], wave, m, l, c, gshift, ginv);
-        if (nt > 8) store_rows<DT, 16, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
-        else if (nt > 4) store_rows<DT, 8, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
-        else if (nt > 2) store_rows<DT, 4, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
-        else if (nt > 1) store_rows<DT, 2, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
-        else if (nt > 0) store_rows<DT, 1, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
-    }
-}
-
-// N > 4096: sweep 1 finds the row maximum and sum with an online update per
-// 4096-column block, sweep 2 recomputes the scores and stores.
-template <int DT, bool F32OUT>
-__global__ __launch_bounds__(kGroupThreads) void wide_kernel(RunArgs a) {
-    __shared__ float sM[2][kWavesPerGroup][16];
-    __shared__ float sL[2][kWavesPerGroup][16];
-    if (!header_ok(a) | !(a.flags & kFlagMfmaOk)) return;
-    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-    const PlanRO pv = plan_ro(a.plan, a.nseg);
-    const int wave = uniform((int)(threadIdx.x >> 6));
-    const int per_head = (int)hdr->totals[kPfxWide];
-    const ConstI32 pfx = pv.pfx[kPfxWide];
-    const int64_t h = blockIdx.y;
-    const float c_raw = a.scale * kLog2e;
-    const float c = c_raw < 0.f ? -c_raw : (c_raw == 0.f ? 1.f : c_raw);   // what prepare_scores leaves
-    int xchg = 0;
-    for (int i = blockIdx.x; i < per_head; i += gridDim.x) {
-        const int g = prefix_search(pfx, a.nseg, i);
-        const int r0 = (i - pfx[g]) * kStripRows;
-        const Seg s = load_seg(pv, g, h, a);
-        const SegRes res = make_res(s, a.A, a.B);
-        f32x4 acc[kMaxTiles];
-        float run_m = -INFINITY, run_l = 0.f;
-        for (int cb = 0; cb < s.N; cb += kSplitCols) {
-            const int c0 = cb + wave * kWaveCols;
-            if (c0 >= s.N) continue;
-            float m, l, cc = c_raw;
-            const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
-            stage_scores<DT, kMaxTiles>(acc, s, res, r0, c0);
-            prepare_scores<kMaxTiles>(acc, nt, s.N, c0, cc);
-            local_softmax<kMaxTiles>(acc, nt, cc, m, l);
-            const float nm = fmaxf(run_m, m);
-            const float nshift = (nm == -INFINITY) ? 0.f : nm;
-            const float f_old = (run_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((run_m - nshift) * c);
-            const float f_new = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m - nshift) * c);
-            run_l = run_l * f_old + l * f_new;
-            run_m = nm;
-        }
-        const int buf = xchg & 1;
-        ++xchg;
-        float gshift, ginv;
-        exchange_row_stats(sM[buf], sL[buf], wave, run_m, run_l, c, gshift, ginv);
-        const float bias = -gshift * c;
-        for (int cb = 0; cb < s.N; cb += kSplitCols) {
-            const int c0 = cb + wave * kWaveCols;
-            if (c0 >= s.N) continue;
-            float cc = c_raw;
-            const int nt = min(kMaxTiles, (s.N - c0 + 15) >> 4);
-            stage_scores<DT, kMaxTiles>(acc, s, res, r0, c0);
-            prepare_scores<kMaxTiles>(acc, nt, s.N, c0, cc);
-#pragma unroll
-            for (int t = 0; t < kMaxTiles; ++t)
-#pragma unroll
-                for (int k = 0; k < 4; ++k) acc[t][k] = __builtin_amdgcn_exp2f(fmaf(acc[t][k], c, bias));
-            store_rows<DT, kMaxTiles, F32OUT>(acc, nt, s, a.out, r0, c0, ginv);
-        }
-    }
-}
-
 // --------------------------------------------------------------------- host
 // With a host copy of the plan summary the grids cover the work exactly and
 // kernels with nothing to do are not launched; without it every kernel is
 // launched with a generous grid and reads the counts from the plan.
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// One call = up to three launches, each taking its own class of segments:
+//   strip kernel    strip-class segments whose B_g fits its LDS window
+//   tile kernel     large segments (see tile_segment())
+//   segment kernel  packs, the element-wise class, and what the two above leave
+// With a host copy of the plan summary the grids cover the work exactly and kernels
+// with nothing to do are not launched; without it all three are launched with
+// generous grids and read everything from the plan.  The first launch reports a
+// plan that does not match the call; the later ones stay quiet.
 template <int DT, bool FUSED, bool F32OUT>
-static int launch_set(const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
-    if (args.H > 65535) return BA_ERR_UNSUPPORTED;      // heads ride on gridDim.y
+static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
+    if (args_in.H > 65535) return BA_ERR_UNSUPPORTED;      // heads ride on gridDim.y
     const int cus = device_cu_count();
-    const bool mfma_ok = args.flags & kFlagMfmaOk;
-    const unsigned H = (unsigned)args.H;
-    // segment kernel: z spreads the 16-row strips (or rows) of the largest segment over workgroups
-    int64_t z = 4;
-    bool seg_work = true;
-    int64_t g_gemm = (int64_t)cus * 8, g_split = (int64_t)cus * 4, g_wide = (int64_t)cus * 4;
-    if (info) {
-        nseg = info->nseg;
-        const int64_t units = mfma_ok && info->slow_items == 0 ? ceil_div(std::min<int64_t>(info->max_M, 256), kStripRows)
-                                                                 : std::min<int64_t>(info->max_M, 4096);
-        z = std::max<int64_t>(1, std::min<int64_t>(64, ceil_div(units, kSegWaves)));
-        seg_work = !mfma_ok || info->strip_items + info->pack_items + info->slow_items > 0;
-        g_gemm = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, ceil_div(info->gemm_items, kSegWaves)) : 0;
-        g_split = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, info->split_items) : 0;
-        g_wide = mfma_ok ? std::min<int64_t>((int64_t)cus * 64, info->wide_items) : 0;
-    }
-    // Strip kernel: with a plan summary, launched when strip-class segments exist; it takes those whose
-    // B_g fits its window, the segment kernel below takes the rest (and is skipped when nothing is left).
-    RunArgs args_rest = args;
-    if (nseg > 0 && mfma_ok && (!info || info->strip_items > 0)) {
+    const bool mfma_ok = args_in.flags & kFlagMfmaOk;
+    const unsigned H = (unsigned)args_in.H;
+    if (info) nseg = info->nseg;
+    if (nseg <= 0) return BA_OK;
+    RunArgs args = args_in;
+
+    const bool strip_work = mfma_ok && (!info || info->strip_items > 0);
+    const bool tile_work = mfma_ok && (!info || info->split_items + info->wide_items + info->strip_rest > 0);
+    const bool seg_work = !mfma_ok || !info || info->pack_items + info->slow_items + info->strip_rest > 0 ||
+                          !(strip_work || tile_work);
+    if (strip_work) args.flags |= kFlagFastStrips;
+    if (tile_work) args.flags |= kFlagTiles;
+
+    if (strip_work) {
         int64_t blocks = kFastBlocks, zf = 2;
         bool lean = false;
         if (info) {
@@ -1030,18 +825,26 @@ static int launch_set(const RunArgs &args, int64_t nseg, const ba_plan_info *inf
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         else
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
-        args_rest.flags |= kFlagFastStrips;
-        if (info && info->strip_rest == 0 && info->pack_items + info->slow_items == 0) seg_work = false;
+        args.flags |= kFlagQuiet;
     }
-    if (nseg > 0 && seg_work) {
-        // LDS window for B_g: whole B_g of the largest strip-class segment if known, else 32 KiB.
-        RunArgs seg_args = args_rest;
-        int64_t blocks = 32;
+    if (tile_work) {
+        const int st = launch_tiles(dtype, FUSED ? 1 : 0, args, nseg, info, stream);
+        if (st != BA_OK) return st;
+        args.flags |= kFlagQuiet;
+    }
+    if (seg_work) {
+        // z spreads the 16-row strips (or rows) of the largest segment over workgroups
+        int64_t z = 4, blocks = 32;
         if (info) {
+            const int64_t units = mfma_ok && info->slow_items == 0 ? ceil_div(std::min<int64_t>(info->max_M, 256), kStripRows)
+                                                                     : std::min<int64_t>(info->max_M, 4096);
+            z = std::max<int64_t>(1, std::min<int64_t>(64, ceil_div(units, kSegWaves)));
+            // LDS window for B_g: whole B_g of the largest strip-class segment if it fits 64 KiB
             const int64_t nt = ceil_div(std::min<int64_t>(std::max<int64_t>(info->max_N, 1), kWaveCols), 16);
             const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
             blocks = std::max<int64_t>(nt, std::min<int64_t>(nt * nks, 64));
         }
+        RunArgs seg_args = args;
         seg_args.lds_blocks = (int)blocks;
         const dim3 grid((unsigned)nseg, H, (unsigned)z);
         const size_t lds_bytes = (size_t)blocks * kLdsBlockBytes;
@@ -1052,14 +855,6 @@ static int launch_set(const RunArgs &args, int64_t nseg, const ba_plan_info *inf
             hipLaunchKernelGGL((segment_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream,
                                seg_args);
     }
-    if (!FUSED && g_gemm > 0)
-        hipLaunchKernelGGL((gemm_large_kernel<DT>), dim3((unsigned)g_gemm, H), dim3(kSegThreads), 0, stream, args);
-    if (FUSED && g_split > 0)
-        hipLaunchKernelGGL((split_kernel<DT, F32OUT>), dim3((unsigned)g_split, H), dim3(kGroupThreads), 0, stream,
-                           args);
-    if (FUSED && g_wide > 0)
-        hipLaunchKernelGGL((wide_kernel<DT, F32OUT>), dim3((unsigned)g_wide, H), dim3(kGroupThreads), 0, stream,
-                           args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
@@ -1067,14 +862,14 @@ int launch_strips(int dtype, int fused, const RunArgs &args, int64_t nseg, const
                   hipStream_t stream) {
     const bool f32out = args.flags & kFlagOutF32;
     if (dtype == BA_F16) {
-        if (!fused) return launch_set<0, false, false>(args, nseg, info, stream);
-        return f32out ? launch_set<0, true, true>(args, nseg, info, stream)
-                      : launch_set<0, true, false>(args, nseg, info, stream);
+        if (!fused) return launch_set<0, false, false>(dtype, args, nseg, info, stream);
+        return f32out ? launch_set<0, true, true>(dtype, args, nseg, info, stream)
+                      : launch_set<0, true, false>(dtype, args, nseg, info, stream);
     }
     if (dtype == BA_BF16) {
-        if (!fused) return launch_set<1, false, false>(args, nseg, info, stream);
-        return f32out ? launch_set<1, true, true>(args, nseg, info, stream)
-                      : launch_set<1, true, false>(args, nseg, info, stream);
+        if (!fused) return launch_set<1, false, false>(dtype, args, nseg, info, stream);
+        return f32out ? launch_set<1, true, true>(dtype, args, nseg, info, stream)
+                      : launch_set<1, true, false>(dtype, args, nseg, info, stream);
     }
     return BA_ERR_UNSUPPORTED;
 }
