@@ -81,7 +81,7 @@ enum SegKind : int32_t {
 
 // Segments the tile kernel takes: N > 256, or strip-class segments too large for the strip
 // kernel's LDS window that have at least one full chunk of columns.
-constexpr int kTileCols = 64;
+constexpr int kTileCols = 128;
 __host__ __device__ inline bool tile_segment(int kind, int N, int K) {
     if (kind == kSegSplit || kind == kSegWide) return true;
     return kind == kSegStrip && !fast_strip_shape(N, K) && N >= kTileCols;
