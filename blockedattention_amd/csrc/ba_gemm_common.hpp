@@ -61,6 +61,67 @@ __device__ __forceinline__ void row16_sum4(float (&x)[4]) { BA_ROT_REDUCE("v_add
 #undef BA_ROT_REDUCE
 #undef BA_ROT_STEP
 
+// Row softmax over values laid out as "lane runs": lane (j = lane%16, rg = lane/16) holds G
+// consecutive columns (index g) of four rows (index e) in acc[g][e]; the sixteen lanes of a row group
+// together hold whole rows.  In: scores, c >= 0 (scale * log2 e), w[g] in {0, 1} = whether the
+// column counts in the row sum (0 for columns a neighbouring lane also holds, or that do not exist;
+// such columns must hold a value that does not exceed the row maximum).  Out: probabilities.
+template <int G>
+__device__ __forceinline__ void softmax_lane_runs(f32x4 (&acc)[G], const float (&w)[G], float c) {
+    float ext[4], sum[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        ext[e] = acc[0][e];
+#pragma unroll
+        for (int g = 1; g + 1 < G; g += 2) ext[e] = max3(ext[e], acc[g][e], acc[g + 1][e]);
+        ext[e] = max3(ext[e], acc[G - 1][e], acc[G - 1][e]);
+    }
+    row16_max4(ext);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float bias = -((__builtin_fabsf(ext[e]) == INFINITY) ? 0.f : ext[e]) * c;
+        sum[e] = 0.f;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float pr = __builtin_amdgcn_exp2f(fmaf(acc[g][e], c, bias));
+            acc[g][e] = pr;
+            sum[e] = fmaf(pr, w[g], sum[e]);
+        }
+    }
+    row16_sum4(sum);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float inv = __builtin_amdgcn_rcpf(sum[e]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) acc[g][e] *= inv;
+    }
+}
+
+// One row (register index e) of a lane's run of G values to memory as the widest stores; the address
+// may have any element alignment.
+template <int DT, int G, bool F32OUT>
+__device__ __forceinline__ void store_run(char *dst, const f32x4 (&acc)[G], int e) {
+    if constexpr (!F32OUT) {
+        uint32_t w[G / 2];
+#pragma unroll
+        for (int k = 0; k < G / 2; ++k) w[k] = Elem<DT>::pack2(acc[2 * k][e], acc[2 * k + 1][e]);
+#pragma unroll
+        for (int k = 0; k + 4 <= G / 2; k += 4)
+            *reinterpret_cast<u32x4_unaligned *>(dst + 4 * k) = u32x4{w[k], w[k + 1], w[k + 2], w[k + 3]};
+        constexpr int kDone = (G / 2) & ~3;
+        if constexpr (((G / 2) & 2) != 0)
+            *reinterpret_cast<u32x2_unaligned *>(dst + 4 * kDone) = u32x2{w[kDone], w[kDone + 1]};
+        if constexpr (((G / 2) & 1) != 0) *reinterpret_cast<u32_unaligned *>(dst + 4 * (G / 2 - 1)) = w[G / 2 - 1];
+    } else {
+#pragma unroll
+        for (int k = 0; k + 4 <= G; k += 4)
+            *reinterpret_cast<f32x4_unaligned *>(dst + 4 * k) =
+                f32x4{acc[k][e], acc[k + 1][e], acc[k + 2][e], acc[k + 3][e]};
+        if constexpr ((G & 2) != 0)
+            *reinterpret_cast<f32x2_unaligned *>(dst + 4 * (G - 2)) = f32x2{acc[G - 2][e], acc[G - 1][e]};
+    }
+}
+
 __device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
     const SegRec r = load_rec(pv.recs, g);   // scalar loads
     Seg s;

@@ -512,28 +512,6 @@ __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, c
 // value by 1 or 0 (w[g]) so overlapped and repeated columns count once; the row
 // maximum needs no mask at all.
 
-// One row of a lane's run (G values scaled by factor) to memory as the widest stores.
-template <int DT, int G, bool F32OUT>
-__device__ __forceinline__ void store_run(char *dst, const f32x4 (&acc)[G], int e) {
-    if (!F32OUT) {
-        uint32_t w[G / 2];
-#pragma unroll
-        for (int k = 0; k < G / 2; ++k) w[k] = Elem<DT>::pack2(acc[2 * k][e], acc[2 * k + 1][e]);
-#pragma unroll
-        for (int k = 0; k + 4 <= G / 2; k += 4)
-            *reinterpret_cast<u32x4_unaligned *>(dst + 4 * k) = u32x4{w[k], w[k + 1], w[k + 2], w[k + 3]};
-        constexpr int kDone = (G / 2) & ~3;
-        if ((G / 2) & 2) *reinterpret_cast<u32x2_unaligned *>(dst + 4 * kDone) = u32x2{w[kDone], w[kDone + 1]};
-        if ((G / 2) & 1) *reinterpret_cast<u32_unaligned *>(dst + 4 * (G / 2 - 1)) = w[G / 2 - 1];
-    } else {
-#pragma unroll
-        for (int k = 0; k + 4 <= G; k += 4)
-            *reinterpret_cast<f32x4_unaligned *>(dst + 4 * k) =
-                f32x4{acc[k][e], acc[k + 1][e], acc[k + 2][e], acc[k + 3][e]};
-        if (G & 2) *reinterpret_cast<f32x2_unaligned *>(dst + 4 * (G - 2)) = f32x2{acc[G - 2][e], acc[G - 1][e]};
-    }
-}
-
 template <int DT, int G, bool FUSED, bool F32OUT>
 __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, unsigned char *lds, int wave,
                                              int first_strip, int strip_step) {
@@ -628,35 +606,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         }
         load_a(strip + strip_step);          // next strip's fragments fly under the softmax and the stores
 
-        if (FUSED) {
-            float ext[4], sum[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                ext[e] = acc[0][e];
-#pragma unroll
-                for (int g = 1; g + 1 < G; g += 2) ext[e] = max3(ext[e], acc[g][e], acc[g + 1][e]);
-                ext[e] = max3(ext[e], acc[G - 1][e], acc[G - 1][e]);
-            }
-            row16_max4(ext);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float bias = -((__builtin_fabsf(ext[e]) == INFINITY) ? 0.f : ext[e]) * c;
-                sum[e] = 0.f;
-#pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const float pr = __builtin_amdgcn_exp2f(fmaf(acc[g][e], c, bias));
-                    acc[g][e] = pr;
-                    sum[e] = fmaf(pr, w[g], sum[e]);
-                }
-            }
-            row16_sum4(sum);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float inv = __builtin_amdgcn_rcpf(sum[e]);
-#pragma unroll
-                for (int g = 0; g < G; ++g) acc[g][e] *= inv;
-            }
-        }
+        if (FUSED) softmax_lane_runs<G>(acc, w, c);
 
         if (owner) {
             const int r0 = strip * kStripRows;

@@ -1,39 +1,59 @@
 // Standalone blocked row softmax: dst row = softmax(scale * src row) for every
 // row of every segment (csrc/cuda/spBlkSoftmax.cu:88-138, 182-269 restated for
-// wave64).  fp32 arithmetic for every dtype, one rounding at the store, no
-// column limit.
+// wave64), and its backward.  fp32 arithmetic for every dtype, one rounding at
+// the store, no column limit.
 //
-// A row is a contiguous run of `cols` elements, and consecutive rows of a
-// segment are contiguous too.  Rows of up to 64*kRegs elements are held in
-// registers by one wavefront (lane-strided, so every load and store of the
-// wavefront is one contiguous 128/256-byte run); longer rows are re-read from
-// the cache hierarchy in three passes.
+// A segment is a contiguous run of rows x cols elements, rows back to back.  The
+// memory pipeline works per lane access, so both kernels move 16 bytes per lane
+// with adjacent lanes on adjacent addresses, at whatever element alignment the
+// rows happen to have:
+//   lane-run kernel  cols <= 256.  Sixteen lanes share a row: lane j owns the G
+//                    consecutive columns [G*j, G*j + G) (G = even tile count
+//                    covering cols), a wavefront takes 16 rows at a time, four per
+//                    instruction -- the layout of the fused strip kernel, with the
+//                    scores loaded instead of computed.  Ragged cols: the lane
+//                    holding the row's end takes the run [cols - G, cols), which
+//                    overlaps its neighbour (both load and store identical values,
+//                    the overlap counts once in the row sum); there are no partial
+//                    loads or stores.
+//   row kernel       cols > 256 (and cols < 2).  One wavefront per row, lane l owns
+//                    the eight columns 8*l + 512*k; rows of up to 4096 columns stay
+//                    in registers, longer rows are re-read in three passes.
 #include <algorithm>
 
-#include "ba_device.hpp"
-#include "ba_host.hpp"
+#include "ba_gemm_common.hpp"
 
 namespace ba {
 
 constexpr int kSoftmaxThreads = 256;
 constexpr int kSoftmaxWaves = kSoftmaxThreads / 64;
-constexpr int kRegs = 16;  // elements per lane kept in registers: rows up to 1024 columns
+constexpr int kRowSteps = 8;      // 512-column steps a row keeps in registers (4096 columns)
+constexpr int kRunCols = 256;     // widest row of the lane-run kernel
 
 template <int DT> struct Io;
 template <> struct Io<BA_F16> {
     typedef uint16_t T;
     static __device__ __forceinline__ float ld(const T *p) { return Elem<0>::to_float(*p); }
     static __device__ __forceinline__ void st(T *p, float v) { *p = Elem<0>::from_float(v); }
+    static __device__ __forceinline__ float lo(uint32_t w) { return Elem<0>::to_float((uint16_t)w); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return Elem<0>::to_float((uint16_t)(w >> 16)); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) { return Elem<0>::pack2(a, b); }
 };
 template <> struct Io<BA_BF16> {
     typedef uint16_t T;
     static __device__ __forceinline__ float ld(const T *p) { return Elem<1>::to_float(*p); }
     static __device__ __forceinline__ void st(T *p, float v) { *p = Elem<1>::from_float(v); }
+    static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) { return Elem<1>::pack2(a, b); }
 };
 template <> struct Io<BA_F32> {
     typedef float T;
     static __device__ __forceinline__ float ld(const T *p) { return *p; }
     static __device__ __forceinline__ void st(T *p, float v) { *p = v; }
+    static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w); }   // unused
+    static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w); }   // unused
+    static __device__ __forceinline__ uint32_t pack(float a, float) { return __builtin_bit_cast(uint32_t, a); }
 };
 
 struct SoftmaxArgs {
@@ -57,8 +77,185 @@ __device__ __forceinline__ int softmax_plan_nseg(const SoftmaxArgs &a) {
     return -1;
 }
 
-// grid (segment, head, z): the workgroup's wavefronts walk the rows of one
-// segment of one head, row r going to wavefront r mod (4 * gridDim.z).
+// ---------------------------------------------------------------- lane runs
+// G consecutive elements of one row from memory into x[g][e] (any element alignment).
+template <int DT, int G>
+__device__ __forceinline__ void load_run(const typename Io<DT>::T *p, f32x4 (&x)[G], int e) {
+    if constexpr (DT == BA_F32) {
+        const float *q = reinterpret_cast<const float *>(p);
+#pragma unroll
+        for (int k = 0; k + 4 <= G; k += 4) {
+            const f32x4 v = *reinterpret_cast<const f32x4_unaligned *>(q + k);
+            x[k][e] = v[0]; x[k + 1][e] = v[1]; x[k + 2][e] = v[2]; x[k + 3][e] = v[3];
+        }
+        if constexpr ((G & 2) != 0) {
+            const f32x2 v = *reinterpret_cast<const f32x2_unaligned *>(q + (G - 2));
+            x[G - 2][e] = v[0]; x[G - 1][e] = v[1];
+        }
+    } else {
+        typedef Io<DT> I;
+        const char *q = reinterpret_cast<const char *>(p);
+        uint32_t w[G / 2];
+#pragma unroll
+        for (int k = 0; k + 4 <= G / 2; k += 4) {
+            const u32x4 v = *reinterpret_cast<const u32x4_unaligned *>(q + 4 * k);
+            w[k] = v[0]; w[k + 1] = v[1]; w[k + 2] = v[2]; w[k + 3] = v[3];
+        }
+        constexpr int kDone = (G / 2) & ~3;
+        if constexpr (((G / 2) & 2) != 0) {
+            const u32x2 v = *reinterpret_cast<const u32x2_unaligned *>(q + 4 * kDone);
+            w[kDone] = v[0]; w[kDone + 1] = v[1];
+        }
+        if constexpr (((G / 2) & 1) != 0) w[G / 2 - 1] = *reinterpret_cast<const u32_unaligned *>(q + 4 * (G / 2 - 1));
+#pragma unroll
+        for (int k = 0; k < G / 2; ++k) { x[2 * k][e] = I::lo(w[k]); x[2 * k + 1][e] = I::hi(w[k]); }
+    }
+}
+
+template <int DT, int G, bool BACKWARD>
+__device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0, int rows, int cols, int first_strip,
+                                             int strip_step) {
+    typedef typename Io<DT>::T T;
+    const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
+    const int J = cols / G, v = cols - G * J;
+    const bool owner = j < J || (j == J && v > 0);
+    const int col0 = j < J ? G * j : cols - G;
+    float w[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) w[g] = (j < J || (j == J && g >= G - v)) ? 1.f : 0.f;
+    const T *src = reinterpret_cast<const T *>(a.src) + seg0 + col0;
+    const T *aux = reinterpret_cast<const T *>(a.aux) + seg0 + col0;
+    T *dst = reinterpret_cast<T *>(a.dst) + seg0 + col0;
+    const float c_signed = a.scale * kLog2e;
+    const float sgn = c_signed < 0.f ? -1.f : 1.f;   // forward works on sgn * x so that the multiplier is >= 0
+    const float c = c_signed * sgn;
+    const int strips = (rows + 15) >> 4;
+    for (int strip = first_strip; strip < strips; strip += strip_step) {
+        // register e of row group rg is row 16*strip + 4*e + rg: an instruction covers four consecutive rows
+        const int r0 = 16 * strip + rg;
+        f32x4 x[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) x[g] = f32x4{-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
+        if (!BACKWARD) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (owner && r0 + 4 * e < rows) load_run<DT, G>(src + (int64_t)(r0 + 4 * e) * cols, x, e);
+            if (sgn < 0.f) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) x[g] = -x[g];
+            }
+            softmax_lane_runs<G>(x, w, c);
+        } else {
+            // dx = scale * (dy - sum(y * dy)) * y; src is the saved forward output here
+            f32x4 dy[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) { x[g] = f32x4{0.f, 0.f, 0.f, 0.f}; dy[g] = x[g]; }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (owner && r0 + 4 * e < rows) {
+                    load_run<DT, G>(src + (int64_t)(r0 + 4 * e) * cols, x, e);
+                    load_run<DT, G>(aux + (int64_t)(r0 + 4 * e) * cols, dy, e);
+                }
+            float dot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int g = 0; g < G; ++g) dot[e] = fmaf(x[g][e] * dy[g][e], w[g], dot[e]);
+            row16_sum4(dot);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int g = 0; g < G; ++g) x[g][e] = a.scale * (dy[g][e] - dot[e]) * x[g][e];
+        }
+        if (owner) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (r0 + 4 * e < rows)
+                    store_run<DT == BA_BF16 ? 1 : 0, G, DT == BA_F32>(
+                        reinterpret_cast<char *>(dst + (int64_t)(r0 + 4 * e) * cols), x, e);
+        }
+    }
+}
+
+// grid (segment, head, z): the wavefronts of the workgroups with the same (segment, head) share the
+// segment's 16-row strips round-robin.
+template <int DT, bool BACKWARD>
+__global__ __launch_bounds__(kSoftmaxThreads) void softmax_runs_kernel(SoftmaxArgs a) {
+    typedef typename Io<DT>::T T;
+    const int nseg = softmax_plan_nseg(a);
+    const int g = blockIdx.x;
+    if (g >= nseg) return;
+    const PlanRO pv = plan_ro(a.plan, nseg);
+    const SegRec rec = load_rec(pv.recs, g);
+    const int rows = rec.M, cols = rec.N;
+    if (cols < 1 || cols > kRunCols || rows < 1) return;
+    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int first = blockIdx.z * kSoftmaxWaves + wave, step = gridDim.z * kSoftmaxWaves;
+    const int64_t seg0 = (int64_t)blockIdx.y * a.Dsrc + rec.offO;
+    if (cols == 1) {
+        // one column: softmax is 1 (NaN where the input is not finite); backward is 0 * (...) likewise
+        const T *src = reinterpret_cast<const T *>(a.src) + seg0;
+        const T *aux = reinterpret_cast<const T *>(a.aux) + seg0;
+        T *dst = reinterpret_cast<T *>(a.dst) + seg0;
+        for (int r = first * 64 + lane_id(); r < rows; r += step * 64) {
+            const float x = Io<DT>::ld(src + r);
+            if (!BACKWARD) {
+                Io<DT>::st(dst + r, fmaf(x, 0.f, 1.f));
+            } else {
+                const float dy = Io<DT>::ld(aux + r);
+                Io<DT>::st(dst + r, a.scale * (dy - x * dy) * x);
+            }
+        }
+        return;
+    }
+    const int tiles = fast_strip_tiles(cols);
+#define BA_RUNS(G_) case G_: softmax_runs<DT, G_, BACKWARD>(a, seg0, rows, cols, first, step); break;
+    switch (tiles) {
+        BA_RUNS(2) BA_RUNS(4) BA_RUNS(6) BA_RUNS(8) BA_RUNS(10) BA_RUNS(12) BA_RUNS(14) BA_RUNS(16)
+        default: break;
+    }
+#undef BA_RUNS
+}
+
+// --------------------------------------------------------------------- rows
+// One wavefront per row; lane l owns columns 8*l .. 8*l+7 of every 512-column step.
+template <int DT>
+__device__ __forceinline__ void load_eight(const typename Io<DT>::T *p, int valid, float fill, float (&x)[8]) {
+    typedef Io<DT> I;
+    if (valid >= 8) {
+        if constexpr (DT == BA_F32) {
+            const f32x4 lo = *reinterpret_cast<const f32x4_unaligned *>(p);
+            const f32x4 hi = *reinterpret_cast<const f32x4_unaligned *>(reinterpret_cast<const float *>(p) + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { x[i] = lo[i]; x[4 + i] = hi[i]; }
+        } else {
+            const u32x4 v = *reinterpret_cast<const u32x4_unaligned *>(p);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { x[2 * i] = I::lo(v[i]); x[2 * i + 1] = I::hi(v[i]); }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = i < valid ? I::ld(p + i) : fill;
+    }
+}
+template <int DT>
+__device__ __forceinline__ void store_eight(typename Io<DT>::T *p, int valid, const float (&x)[8]) {
+    typedef Io<DT> I;
+    if (valid >= 8) {
+        if constexpr (DT == BA_F32) {
+            *reinterpret_cast<f32x4_unaligned *>(p) = f32x4{x[0], x[1], x[2], x[3]};
+            *reinterpret_cast<f32x4_unaligned *>(reinterpret_cast<float *>(p) + 4) = f32x4{x[4], x[5], x[6], x[7]};
+        } else {
+            *reinterpret_cast<u32x4_unaligned *>(p) =
+                u32x4{I::pack(x[0], x[1]), I::pack(x[2], x[3]), I::pack(x[4], x[5]), I::pack(x[6], x[7])};
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i < valid) I::st(p + i, x[i]);
+    }
+}
+
 template <int DT, bool BACKWARD>
 __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxArgs a) {
     typedef typename Io<DT>::T T;
@@ -68,7 +265,7 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
     const PlanRO pv = plan_ro(a.plan, nseg);
     const SegRec rec = load_rec(pv.recs, g);
     const int rows = rec.M, cols = rec.N;
-    if (cols < 1) return;
+    if (cols <= kRunCols) return;                       // the lane-run kernel's
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int lane = lane_id();
     const int first = blockIdx.z * kSoftmaxWaves + wave, stride = gridDim.z * kSoftmaxWaves;
@@ -76,39 +273,51 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
     const T *src = reinterpret_cast<const T *>(a.src) + seg0;
     const T *aux = reinterpret_cast<const T *>(a.aux) + seg0;
     T *dst = reinterpret_cast<T *>(a.dst) + seg0;
-    float c = a.scale * kLog2e;
-    const float sgn = c < 0.f ? -1.f : 1.f;  // forward works on sgn*x so the multiplier is >= 0
-    c *= sgn;
+    const float c_signed = a.scale * kLog2e;
+    const float sgn = c_signed < 0.f ? -1.f : 1.f;
+    const float c = c_signed * sgn;
+    const int steps = (cols + 511) >> 9;
 
     for (int r = first; r < rows; r += stride) {
         const int64_t e0 = (int64_t)r * cols;
         const T *x = src + e0;
         T *y = dst + e0;
         if (!BACKWARD) {
-            if (cols <= 64 * kRegs) {
-                float v[kRegs];
-                float mx = -INFINITY;
+            if (steps <= kRowSteps) {
+                float v[kRowSteps][8];
+                float mx = -3.0e38f;
 #pragma unroll
-                for (int j = 0; j < kRegs; ++j) {
-                    const int col = lane + 64 * j;
-                    v[j] = (col < cols) ? sgn * Io<DT>::ld(x + col) : -INFINITY;
-                    mx = fmaxf(mx, v[j]);
+                for (int k = 0; k < kRowSteps; ++k) {
+                    if (k < steps) {
+                        const int col = 512 * k + 8 * lane;
+                        load_eight<DT>(x + col, cols - col, -3.0e38f * sgn, v[k]);
+#pragma unroll
+                        for (int i = 0; i < 8; i += 2) mx = max3(mx, sgn * v[k][i], sgn * v[k][i + 1]);
+                    }
                 }
                 mx = wave_max(mx);
-                const float bias = -((mx == -INFINITY) ? 0.f : mx) * c;
+                const float bias = -((__builtin_fabsf(mx) == INFINITY) ? 0.f : mx) * c;
                 float sum = 0.f;
 #pragma unroll
-                for (int j = 0; j < kRegs; ++j) {
-                    const int col = lane + 64 * j;
-                    v[j] = (col < cols) ? __builtin_amdgcn_exp2f(fmaf(v[j], c, bias)) : 0.f;
-                    sum += v[j];
+                for (int k = 0; k < kRowSteps; ++k) {
+                    if (k < steps) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            v[k][i] = __builtin_amdgcn_exp2f(fmaf(sgn * v[k][i], c, bias));
+                            sum += v[k][i];
+                        }
+                    }
                 }
                 sum = wave_sum(sum);
-                const float inv = 1.f / sum;
+                const float inv = __builtin_amdgcn_rcpf(sum);
 #pragma unroll
-                for (int j = 0; j < kRegs; ++j) {
-                    const int col = lane + 64 * j;
-                    if (col < cols) Io<DT>::st(y + col, v[j] * inv);
+                for (int k = 0; k < kRowSteps; ++k) {
+                    if (k < steps) {
+                        const int col = 512 * k + 8 * lane;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) v[k][i] *= inv;
+                        store_eight<DT>(y + col, cols - col, v[k]);
+                    }
                 }
             } else {
                 float mx = -INFINITY;
@@ -127,28 +336,22 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
         } else {
             // dx = scale * (dy - sum(y * dy)) * y; x is the saved forward output here.
             const T *dy = aux + e0;
-            if (cols <= 64 * kRegs) {
-                float yv[kRegs], gv[kRegs];
-                float dot = 0.f;
+            float dot = 0.f;
+            for (int col = 8 * lane; col < cols; col += 512) {
+                float yv[8], gv[8];
+                load_eight<DT>(x + col, cols - col, 0.f, yv);
+                load_eight<DT>(dy + col, cols - col, 0.f, gv);
 #pragma unroll
-                for (int j = 0; j < kRegs; ++j) {
-                    const int col = lane + 64 * j;
-                    yv[j] = (col < cols) ? Io<DT>::ld(x + col) : 0.f;
-                    gv[j] = (col < cols) ? Io<DT>::ld(dy + col) : 0.f;
-                    dot = fmaf(yv[j], gv[j], dot);
-                }
-                dot = wave_sum(dot);
+                for (int i = 0; i < 8; ++i) dot = fmaf(yv[i], gv[i], dot);
+            }
+            dot = wave_sum(dot);
+            for (int col = 8 * lane; col < cols; col += 512) {
+                float yv[8], gv[8];
+                load_eight<DT>(x + col, cols - col, 0.f, yv);
+                load_eight<DT>(dy + col, cols - col, 0.f, gv);
 #pragma unroll
-                for (int j = 0; j < kRegs; ++j) {
-                    const int col = lane + 64 * j;
-                    if (col < cols) Io<DT>::st(y + col, a.scale * (gv[j] - dot) * yv[j]);
-                }
-            } else {
-                float dot = 0.f;
-                for (int col = lane; col < cols; col += 64) dot = fmaf(Io<DT>::ld(x + col), Io<DT>::ld(dy + col), dot);
-                dot = wave_sum(dot);
-                for (int col = lane; col < cols; col += 64)
-                    Io<DT>::st(y + col, a.scale * (Io<DT>::ld(dy + col) - dot) * Io<DT>::ld(x + col));
+                for (int i = 0; i < 8; ++i) yv[i] = a.scale * (gv[i] - dot) * yv[i];
+                store_eight<DT>(y + col, cols - col, yv);
             }
         }
     }
@@ -157,14 +360,27 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
 template <int DT, bool BACKWARD>
 static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
     if (args.H > 65535) return BA_ERR_UNSUPPORTED;      // heads ride on gridDim.y
-    int64_t z = 8;
+    const int cus = device_cu_count();
+    // lane-run kernel: z spreads the 16-row strips over workgroups when there are few (segment, head) pairs
+    int64_t z_runs = 4, z_rows = 8;
+    bool rows_work = true;
     if (info) {
         nseg = info->nseg;
-        z = std::max<int64_t>(1, std::min<int64_t>(64, (info->max_M + 4 * kSoftmaxWaves - 1) / (4 * kSoftmaxWaves)));
+        const int64_t groups = (((int64_t)info->max_M + 15) / 16 + kSoftmaxWaves - 1) / kSoftmaxWaves;
+        const int64_t want = ((int64_t)cus * 8 + nseg * args.H - 1) / std::max<int64_t>(1, nseg * args.H);
+        z_runs = std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
+        rows_work = info->max_N > kRunCols;
+        // row kernel: about four workgroups' worth of rows in flight per compute unit, never more than one
+        // wavefront per row
+        z_rows = std::max<int64_t>(1, std::min<int64_t>(4 * want, (info->max_M + kSoftmaxWaves - 1) / kSoftmaxWaves));
     }
     if (nseg <= 0) return BA_OK;
-    hipLaunchKernelGGL((softmax_rows_kernel<DT, BACKWARD>), dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z),
+    hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD>), dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs),
                        dim3(kSoftmaxThreads), 0, stream, args);
+    if (rows_work)
+        hipLaunchKernelGGL((softmax_rows_kernel<DT, BACKWARD>),
+                           dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z_rows), dim3(kSoftmaxThreads), 0, stream,
+                           args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
