@@ -40,6 +40,9 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-others", action="store_true", help="skip the other configurations")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="run only a plain device copy of 64 MiB, 10 times: the known-size kernel against which "
+                        "rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled")
     return p.parse_args()
 
 
@@ -217,6 +220,14 @@ def main():
         return 2
     capi.load()
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.arange(16 << 20, dtype=torch.float32, device=dev)          # 64 MiB
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4, "launches": 10}))
+        return 0
     case = Case(args.config, dev)
     worst = case.check()
     fig = case.gpu_figures(args.steps, args.warmup)
@@ -231,7 +242,7 @@ def main():
         "config": {"workload": w.name, "segments": w.nseg, "heads": w.heads, "seed": 0,
                    "flops": w.flops, "pair_bytes": w.pair_bytes()},
         "roofline": {"bound": "hbm", "achieved": fig["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": fig["hbm_frac"], "traffic": None, "kernel": "ba::segment_kernel (fused GEMM+softmax)",
+                     "frac": fig["hbm_frac"], "traffic": None, "kernel": "ba::strip_kernel (fused GEMM+softmax)",
                      "kernel_us": fig["kernel_us"], "mfma_frac": fig["mfma_frac"], "TFLOPs": fig["TFLOPs"]},
         "parity_max_abs_err": worst,
         "detail": fig,

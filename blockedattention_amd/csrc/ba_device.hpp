@@ -108,7 +108,7 @@ typedef const __attribute__((address_space(4))) PlanHeader *ConstHdr;
 struct PlanRO {
     ConstHdr hdr;
     ConstSeg recs;
-    ConstI32 pfx[kNumPrefix];
+    ConstSeg list[kNumLists];
 };
 
 __device__ __forceinline__ PlanRO plan_ro(const void *buf, int nseg) {
@@ -117,7 +117,7 @@ __device__ __forceinline__ PlanRO plan_ro(const void *buf, int nseg) {
     uintptr_t p = (uintptr_t)buf;
     v.hdr = (ConstHdr)p; p += sizeof(PlanHeader);
     v.recs = (ConstSeg)p; p += cap * sizeof(SegRec);
-    for (int i = 0; i < kNumPrefix; ++i) { v.pfx[i] = (ConstI32)p; p += (cap + 4) * sizeof(int32_t); }
+    for (int i = 0; i < kNumLists; ++i) { v.list[i] = (ConstSeg)p; p += cap * sizeof(SegRec); }
     return v;
 }
 
@@ -127,8 +127,7 @@ __device__ __forceinline__ SegRec load_rec(ConstSeg recs, int g) {
     const ConstI32 w = (ConstI32)(recs + g);
     SegRec r;
     r.off1 = q[0]; r.off2 = q[1]; r.offO = q[2];
-    r.M = w[6]; r.N = w[7]; r.K = w[8]; r.packLen = w[9]; r.kind = w[10];
-    r.pad_ = 0;
+    r.M = w[6]; r.N = w[7]; r.K = w[8]; r.packLen = w[9]; r.kind = w[10]; r.index = w[11];
     return r;
 }
 

@@ -8,6 +8,7 @@ namespace ba {
 
 struct Seg {
     int M, N, K;
+    int kind, index, packLen;   // SegKind, segment index g, pack length (leaders)
     int64_t a, b, o;  // element offsets of the segment inside A, B, out (head included)
 };
 
@@ -126,6 +127,25 @@ __device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, cons
     const SegRec r = load_rec(pv.recs, g);   // scalar loads
     Seg s;
     s.M = r.M; s.N = r.N; s.K = r.K;
+    s.kind = r.kind; s.index = r.index; s.packLen = r.packLen;
+    s.a = h * a.Dm1 + r.off1;
+    s.b = h * a.Dm2 + r.off2;
+    s.o = h * a.Dout + r.offO;
+    return s;
+}
+
+// Segment of a workgroup: entry `slot` of the launch's work list (a compacted copy of the records), or
+// segment `slot` itself when the launch walks every segment.  The record load does not wait for the list
+// length: slots never exceed the arrays.  valid = false past the end of the list.
+__device__ __forceinline__ Seg load_listed(const PlanRO &pv, int slot, int64_t h, const RunArgs &a, bool &valid) {
+    const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+    const int count = a.list < 0 ? a.nseg : (int)hdr->totals[a.list < 0 ? 0 : a.list];
+    // the lists follow the per-segment records back to back, cap records each: list -1 is the records themselves
+    const SegRec r = load_rec(pv.recs + (int64_t)(a.list + 1) * plan_cap(a.nseg), slot);
+    valid = slot < count;
+    Seg s;
+    s.M = r.M; s.N = r.N; s.K = r.K;
+    s.kind = r.kind; s.index = r.index; s.packLen = r.packLen;
     s.a = h * a.Dm1 + r.off1;
     s.b = h * a.Dm2 + r.off2;
     s.o = h * a.Dout + r.offO;

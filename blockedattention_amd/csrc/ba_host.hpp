@@ -13,8 +13,6 @@ enum RunFlags : int {
     kFlagTranspose2 = 2,   // B segments stored K x N
     kFlagMfmaOk = 4,       // layouts, base pointers and head strides allow 16-byte operand loads
     kFlagOutF32 = 8,       // fused path writes fp32 probabilities
-    kFlagFastStrips = 16,  // the strip kernel runs in the same call and takes the segments that fit its window
-    kFlagTiles = 32,       // the tile kernel runs in the same call and takes the large segments
     kFlagQuiet = 64        // an earlier launch of the same call reports a plan that does not match
 };
 
@@ -26,7 +24,8 @@ struct RunArgs {
     int64_t H, Dm1, Dm2, Dout;
     float scale;
     int flags;
-    int lds_blocks;   // 1 KiB operand blocks of dynamic LDS given to the segment kernel
+    int lds_blocks;   // 1 KiB operand blocks of dynamic LDS given to the segment / strip kernel
+    int list;         // work list the launch walks (PrefixKind), or -1: every segment, by block index
     int nseg;         // segment count the plan was built for (checked against the plan)
 };
 
@@ -37,8 +36,8 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
 // info: optional host copy of the plan summary (from ba_plan_read), or nullptr.
 int launch_strips(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
                   hipStream_t stream);
-// The tile kernel over the large segments (see tile_segment()).
-int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
+// The tile kernel over the large segments (see tile_segment()); slots = length of its work list (or nseg).
+int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                  hipStream_t stream);
 int launch_gemm_f32(const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,

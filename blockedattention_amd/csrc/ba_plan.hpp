@@ -3,7 +3,7 @@
 //
 //   PlanHeader                    (256 bytes)
 //   SegRec recs[cap]              one 48-byte record per segment: offsets and shape
-//   int32 prefix arrays, each [cap+4]   scanned work-item counts, one array per kind
+//   SegRec lists[4][cap]          the records of each launch class once more, compacted (work lists)
 //
 // cap = nseg rounded up so that every array starts 16-byte aligned.  The
 // compute kernels read the plan through scalar loads (it is never written
@@ -21,27 +21,44 @@ constexpr int kWavesPerGroup = 16;
 constexpr int kSplitCols = kWaveCols * kWavesPerGroup;  // 4096: columns one workgroup keeps in registers
 constexpr int kPackDim = 16;      // a pack of tiny segments fits one 16x16 MFMA tile
 
-// Strip-class segments whose whole B_g fits the strip kernel's LDS window: G =
-// the even tile count covering N, G * ceil(K/32) operand blocks of 1 KiB.
+// Strip-class segments whose whole B_g fits the strip kernel's LDS window: G = the
+// even tile count covering N, G * ceil(K/32) operand blocks of 1 KiB.  Segments
+// needing up to kFastBlocks blocks run in the main launch; those needing up to
+// kBigBlocks run in a second launch with a larger window (fewer resident
+// workgroups, so it is kept apart from the many small segments).
 constexpr int kFastBlocks = 32;
+constexpr int kBigBlocks = 64;
 constexpr int kFastSteps = 4;     // k-steps of 32 whose A fragments a wavefront holds
 __host__ __device__ inline int fast_strip_tiles(int N) { return 2 * ((N + 31) >> 5); }
-__host__ __device__ inline bool fast_strip_shape(int N, int K) {
+// LDS blocks the strip kernel needs for an N x K operand, or 0 if the shape is not its kind.
+__host__ __device__ inline int strip_blocks(int N, int K) {
     const int nks = (K + 31) >> 5;
-    return N >= 2 && N <= kWaveCols && nks >= 1 && nks <= kFastSteps && fast_strip_tiles(N) * nks <= kFastBlocks;
+    if (N < 2 || N > kWaveCols || nks < 1 || nks > kFastSteps) return 0;
+    return fast_strip_tiles(N) * nks;
+}
+__host__ __device__ inline bool fast_strip_shape(int N, int K) {
+    const int b = strip_blocks(N, K);
+    return b >= 1 && b <= kBigBlocks;
 }
 
-// Kinds of scanned work-item counts.  Every kind except kPfxRows and kPfxSlow
-// counts aligned segments only (see below).
+// What the scheduler scans per segment.  The first four are 0/1 class flags whose
+// scan compacts the segment indices into one work list per launch (the arrays of
+// the plan hold those lists); the others are work-item counts of which only the
+// totals are kept (plan summary).
 enum PrefixKind {
-    kPfxGemm = 0,   // GEMM only, N > 256: ceil(M/16) * ceil(N/256) per segment
-    kPfxStrip = 1,  // fused, N <= 256 and not packed: ceil(M/16)
-    kPfxSplit = 2,  // fused, 256 < N <= 4096: ceil(M/16)
-    kPfxWide = 3,   // fused, N > 4096: ceil(M/16)
-    kPfxRows = 4,   // softmax: M rows
-    kPfxPack = 5,   // 1 for the first segment of a pack of tiny segments, else 0
-    kPfxSlow = 6,   // ceil(M/16) for segments the 16-byte operand loads cannot serve
-    kNumPrefix = 7
+    kListSmall = 0,  // strip-class segments for the strip kernel's main launch (<= kFastBlocks LDS blocks)
+    kListBig = 1,    // strip-class segments for its second launch (<= kBigBlocks)
+    kListTile = 2,   // segments of the tile kernel
+    kListRest = 3,   // everything else that has work: pack leaders, element-wise class, leftovers
+    kNumLists = 4,
+    kPfxGemm = 4,   // GEMM only, N > 256: ceil(M/16) * ceil(N/256) per segment
+    kPfxStrip = 5,  // fused, N <= 256 and not packed: ceil(M/16)
+    kPfxSplit = 6,  // fused, 256 < N <= 4096: ceil(M/16)
+    kPfxWide = 7,   // fused, N > 4096: ceil(M/16)
+    kPfxRows = 8,   // softmax: M rows
+    kPfxPack = 9,   // 1 for the first segment of a pack of tiny segments, else 0
+    kPfxSlow = 10,  // ceil(M/16) for segments the 16-byte operand loads cannot serve
+    kNumPrefix = 11
 };
 
 // A segment is "aligned" when K % 8 == 0 and its A and B offsets are multiples
@@ -57,12 +74,11 @@ struct PlanHeader {
     int32_t kind;            // 0 = GEMM plan, 1 = softmax plan
     int64_t Dm1, Dm2, Dout;
     int64_t total_rows;
-    int64_t totals[8];       // last entry of each prefix array
+    int64_t totals[12];      // totals of the scanned quantities (PrefixKind)
     int32_t max_M, max_N, max_K;
     int32_t bad_segments;
     int32_t run_errors;      // bumped by kernels that refuse to run
-    int32_t strip_rest;      // strip-class segments that do not fit the strip kernel's LDS window
-    int32_t pad_[30];
+    int32_t pad_[23];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 
@@ -87,6 +103,18 @@ __host__ __device__ inline bool tile_segment(int kind, int N, int K) {
     return kind == kSegStrip && !fast_strip_shape(N, K) && N >= kTileCols;
 }
 
+// Launch class (work list) of a segment of a GEMM plan, or -1 for none.
+__host__ __device__ inline int launch_class(int kind, int M, int N, int K) {
+    if (kind == kSegEmpty || kind == kSegPackFollow || M < 1 || N < 1) return -1;
+    if (kind == kSegStrip) {
+        const int b = strip_blocks(N, K);
+        if (b >= 1 && b <= kFastBlocks) return kListSmall;
+        if (b > kFastBlocks && b <= kBigBlocks) return kListBig;
+    }
+    if (tile_segment(kind, N, K)) return kListTile;
+    return kListRest;
+}
+
 // Everything a kernel needs to know about one segment, in one aligned record
 // (three 16-byte scalar loads).
 struct alignas(16) SegRec {
@@ -94,19 +122,19 @@ struct alignas(16) SegRec {
     int32_t M, N, K;
     int32_t packLen;            // > 0: first segment of a pack of this many segments
     int32_t kind;               // SegKind
-    int32_t pad_;
+    int32_t index;              // the segment's index g (records are also kept compacted per launch class)
 };
 static_assert(sizeof(SegRec) == 48, "SegRec must stay 48 bytes");
 
 struct PlanView {
     PlanHeader *hdr;
     SegRec *recs;
-    int32_t *pfx[kNumPrefix];
+    SegRec *list[kNumLists];    // records of one launch class, compacted, in segment order
 };
 
 __host__ __device__ inline size_t plan_bytes_for(int64_t nseg) {
     const size_t cap = (size_t)plan_cap(nseg);
-    return sizeof(PlanHeader) + cap * sizeof(SegRec) + kNumPrefix * (cap + 4) * sizeof(int32_t);
+    return sizeof(PlanHeader) + (1 + kNumLists) * cap * sizeof(SegRec);
 }
 
 __host__ __device__ inline PlanView plan_view(void *buf, int64_t nseg) {
@@ -115,7 +143,7 @@ __host__ __device__ inline PlanView plan_view(void *buf, int64_t nseg) {
     char *p = (char *)buf;
     v.hdr = (PlanHeader *)p; p += sizeof(PlanHeader);
     v.recs = (SegRec *)p; p += cap * sizeof(SegRec);
-    for (int i = 0; i < kNumPrefix; ++i) { v.pfx[i] = (int32_t *)p; p += (cap + 4) * sizeof(int32_t); }
+    for (int i = 0; i < kNumLists; ++i) { v.list[i] = (SegRec *)p; p += cap * sizeof(SegRec); }
     return v;
 }
 

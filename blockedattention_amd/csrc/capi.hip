@@ -93,7 +93,10 @@ __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_pla
     info->max_M = h.max_M; info->max_N = h.max_N; info->max_K = h.max_K;
     info->bad_segments = h.bad_segments;
     info->run_errors = h.run_errors;
-    info->strip_rest = h.strip_rest;
+    info->list_small = (int32_t)h.totals[kListSmall];
+    info->list_big = (int32_t)h.totals[kListBig];
+    info->list_tile = (int32_t)h.totals[kListTile];
+    info->list_rest = (int32_t)h.totals[kListRest];
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 
@@ -105,7 +108,7 @@ __attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_p
     if (!plan || nseg < 0 || nseg > (int64_t(1) << 30) || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
     if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
     if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0, 0, (int)nseg};
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, 1.0f, 0, 0, 0, (int)nseg};
     if (transpose1) args.flags |= kFlagTranspose1;
     if (transpose2) args.flags |= kFlagTranspose2;
     args.flags |= mfma_flag(args);
@@ -144,7 +147,7 @@ __attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_
     if (out_dtype != dtype && out_dtype != BA_F32) return BA_ERR_UNSUPPORTED;
     if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
     if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, (int)nseg};
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, 0, (int)nseg};
     args.flags |= mfma_flag(args);
     if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
     return launch_strips(dtype, 1, args, nseg, info, (hipStream_t)stream);

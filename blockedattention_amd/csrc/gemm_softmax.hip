@@ -659,23 +659,23 @@ __device__ __forceinline__ void strips_exact_dispatch(int tiles, const Seg &s, c
 template <int DT, bool FUSED, bool F32OUT, int MAXNT>
 __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kernel(RunArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-    const int g = blockIdx.x;
-    if (g >= a.nseg) return;
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int64_t h = blockIdx.y;
-    // Header and segment record are fetched together; nothing waits on the header alone.
     const bool ok = header_ok(a);
-    const Seg s = load_seg(pv, g, h, a);
-    const int kind = pv.recs[g].kind;
+    bool valid;
+    const Seg s = load_listed(pv, blockIdx.x, h, a, valid);
     if (!ok) {
         if (!(a.flags & kFlagQuiet)) report_mismatch(a);
         return;
     }
+    if (!valid) return;
+    const int g = s.index;
+    const int kind = s.kind;
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int first = blockIdx.z * kSegWaves + wave, stride = gridDim.z * kSegWaves;
     const bool mfma_ok = (a.flags & kFlagMfmaOk) != 0;
     if (kind == kSegEmpty) return;
-    if (mfma_ok && (a.flags & kFlagTiles) && tile_segment(kind, s.N, s.K)) return;
+    if (mfma_ok && a.list < 0 && launch_class(kind, s.M, s.N, s.K) != kListRest) return;   // another kernel's
     if (!mfma_ok || kind == kSegSlow) {
         // Element-wise path.  With MFMA ruled out for the whole launch this also
         // covers the segments the list kernels would have taken.
@@ -683,7 +683,6 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
         return;
     }
     if (kind == kSegStrip) {
-        if ((a.flags & kFlagFastStrips) && fast_strip_shape(s.N, s.K) && fast_strip_tiles(s.N) <= MAXNT) return;
         // One strip per wavefront; blockIdx.z selects the group of kSegWaves strips.
         const int strips = (s.M + kStripRows - 1) / kStripRows;
         const int nt = (s.N + 15) >> 4;
@@ -694,7 +693,7 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
                                                         strip < strips, wave, kSegWaves);
         }
     } else if (kind == kSegPackLead) {
-        if (first == 0) wave_pack<DT, FUSED, F32OUT>(pv, g, pv.recs[g].packLen, h, a);
+        if (first == 0) wave_pack<DT, FUSED, F32OUT>(pv, g, s.packLen, h, a);
     }
 }
 
@@ -704,19 +703,21 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
 template <int DT, bool FUSED, bool F32OUT, int MAXNT>
 __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(RunArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-    const int g = blockIdx.x;
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int64_t h = blockIdx.y;
+    // header and record are fetched together; nothing waits on the header alone
     const bool ok = header_ok(a);
-    const Seg s = load_seg(pv, g, h, a);
-    const int kind = pv.recs[g].kind;
+    bool valid;
+    const Seg s = load_listed(pv, blockIdx.x, h, a, valid);
     if (!ok) {
         if (!(a.flags & kFlagQuiet)) report_mismatch(a);
         return;
     }
-    if (kind != kSegStrip) return;
+    if (!valid) return;
     const int tiles = fast_strip_tiles(s.N);
-    if (!fast_strip_shape(s.N, s.K) | (tiles > MAXNT)) return;
+    const int need = strip_blocks(s.N, s.K);
+    // the lists hold only segments of this kernel; the checks guard against a launch that does not match
+    if ((s.kind != kSegStrip) | (need < 1) | (need > a.lds_blocks) | (tiles > MAXNT)) return;
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int first = blockIdx.z * kSegWaves + wave, step = gridDim.z * kSegWaves;
     if ((int)blockIdx.z * kSegWaves * kStripRows >= s.M) return;   // no strip for this workgroup
@@ -729,14 +730,14 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
 // launched with a generous grid and reads the counts from the plan.
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// One call = up to three launches, each taking its own class of segments:
-//   strip kernel    strip-class segments whose B_g fits its LDS window
+// One call = up to four launches, each walking its own work list of the plan:
+//   strip kernel    strip-class segments whose B_g fits its LDS window (main launch: up to 32 KiB;
+//                   second launch: up to 64 KiB, fewer resident workgroups)
 //   tile kernel     large segments (see tile_segment())
-//   segment kernel  packs, the element-wise class, and what the two above leave
-// With a host copy of the plan summary the grids cover the work exactly and kernels
-// with nothing to do are not launched; without it all three are launched with
-// generous grids and read everything from the plan.  The first launch reports a
-// plan that does not match the call; the later ones stay quiet.
+//   segment kernel  packs, the element-wise class, and what the others leave
+// With a host copy of the plan summary the grids are exactly the list lengths and empty lists are not
+// launched; without it every kernel is launched over nseg slots and reads its list length from the plan.
+// The first launch reports a plan that does not match the call; the later ones stay quiet.
 template <int DT, bool FUSED, bool F32OUT>
 static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
     if (args_in.H > 65535) return BA_ERR_UNSUPPORTED;      // heads ride on gridDim.y
@@ -746,43 +747,45 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     if (info) nseg = info->nseg;
     if (nseg <= 0) return BA_OK;
     RunArgs args = args_in;
-
-    const bool strip_work = mfma_ok && (!info || info->strip_items > 0);
-    const bool tile_work = mfma_ok && (!info || info->split_items + info->wide_items + info->strip_rest > 0);
-    const bool seg_work = !mfma_ok || !info || info->pack_items + info->slow_items + info->strip_rest > 0 ||
-                          !(strip_work || tile_work);
-    if (strip_work) args.flags |= kFlagFastStrips;
-    if (tile_work) args.flags |= kFlagTiles;
-
-    if (strip_work) {
-        int64_t blocks = kFastBlocks, zf = 2;
-        bool lean = false;
-        if (info) {
+    const int64_t n_small = !mfma_ok ? 0 : info ? info->list_small : nseg;
+    const int64_t n_big = !mfma_ok ? 0 : info ? info->list_big : nseg;
+    const int64_t n_tile = !mfma_ok ? 0 : info ? info->list_tile : nseg;
+    const int64_t n_rest = !mfma_ok ? nseg : info ? info->list_rest : nseg;
+    const bool lean = info && info->max_N <= 128;
+    // z: enough workgroups to fill the machine, at most one per kSegWaves strips of the tallest segment
+    auto strip_z = [&](int64_t slots) {
+        if (!info) return (int64_t)2;
+        const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(info->max_M, 1), kStripRows), kSegWaves);
+        const int64_t want = ceil_div((int64_t)cus * 8, std::max<int64_t>(1, slots * (int64_t)H));
+        return std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
+    };
+    for (int pass = 0; pass < 2; ++pass) {
+        const int64_t slots = pass == 0 ? n_small : n_big;
+        if (slots <= 0) continue;
+        RunArgs fa = args;
+        fa.list = pass == 0 ? kListSmall : kListBig;
+        fa.lds_blocks = pass == 0 ? kFastBlocks : kBigBlocks;
+        if (info && pass == 0) {
             const int64_t nt = fast_strip_tiles((int)std::min<int64_t>(std::max<int64_t>(info->max_N, 1), kWaveCols));
             const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
-            blocks = std::min<int64_t>(kFastBlocks, nt * nks);
-            lean = info->max_N <= 128;
-            // enough workgroups to fill the machine, at most one per kSegWaves strips
-            const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(info->max_M, 1), kStripRows), kSegWaves);
-            const int64_t want = ceil_div((int64_t)cus * 8, std::max<int64_t>(1, nseg * (int64_t)H));
-            zf = std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
+            fa.lds_blocks = (int)std::min<int64_t>(kFastBlocks, nt * nks);
         }
-        RunArgs fa = args;
-        fa.lds_blocks = (int)blocks;
-        const dim3 grid((unsigned)nseg, H, (unsigned)zf);
-        const size_t lds_bytes = (size_t)blocks * kLdsBlockBytes;
+        const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots));
+        const size_t lds_bytes = (size_t)fa.lds_blocks * kLdsBlockBytes;
         if (lean)
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         else
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         args.flags |= kFlagQuiet;
     }
-    if (tile_work) {
-        const int st = launch_tiles(dtype, FUSED ? 1 : 0, args, nseg, info, stream);
+    if (n_tile > 0) {
+        RunArgs ta = args;
+        ta.list = kListTile;
+        const int st = launch_tiles(dtype, FUSED ? 1 : 0, ta, n_tile, info, stream);
         if (st != BA_OK) return st;
         args.flags |= kFlagQuiet;
     }
-    if (seg_work) {
+    if (n_rest > 0) {
         // z spreads the 16-row strips (or rows) of the largest segment over workgroups
         int64_t z = 4, blocks = 32;
         if (info) {
@@ -795,10 +798,11 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
             blocks = std::max<int64_t>(nt, std::min<int64_t>(nt * nks, 64));
         }
         RunArgs seg_args = args;
+        seg_args.list = mfma_ok ? kListRest : -1;
         seg_args.lds_blocks = (int)blocks;
-        const dim3 grid((unsigned)nseg, H, (unsigned)z);
+        const dim3 grid((unsigned)n_rest, H, (unsigned)z);
         const size_t lds_bytes = (size_t)blocks * kLdsBlockBytes;
-        if (info && info->max_N <= 128)
+        if (lean)
             hipLaunchKernelGGL((segment_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream,
                                seg_args);
         else

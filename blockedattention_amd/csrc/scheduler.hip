@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
     __shared__ __attribute__((aligned(16))) int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads];
     __shared__ int32_t sPack[kSchedThreads];
-    __shared__ int32_t sRed[kSchedWaves][5];
+    __shared__ int32_t sRed[kSchedWaves][4];
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6), lane = lane_id();
@@ -96,8 +96,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     PlanView pv = plan_view(a.plan, nseg);
 
     int64_t base64[3] = {0, 0, 0};
-    int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0};
-    int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0, nrest = 0;
+    int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
 
     for (int64_t chunk = 0; chunk < nseg || chunk == 0; chunk += kSchedThreads) {
@@ -179,7 +179,16 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         const int32_t chunks = (ni + kWaveCols - 1) / kWaveCols;
         const bool packed = pack != 0;
         const bool mfma_ok = aligned && !packed;
+        const int32_t seg_kind = strips == 0 ? kSegEmpty
+                                 : !aligned ? kSegSlow
+                                 : pack > 0 ? kSegPackLead
+                                 : pack < 0 ? kSegPackFollow
+                                 : ni <= kWaveCols ? kSegStrip
+                                 : ni <= kSplitCols ? kSegSplit : kSegWide;
+        const int cls = a.kind == 0 ? launch_class(seg_kind, mi, ni, ki) : -1;
         int32_t v32[kNumPrefix], t32[kNumPrefix];
+#pragma unroll
+        for (int q = 0; q < kNumLists; ++q) v32[q] = cls == q ? 1 : 0;
         v32[kPfxGemm] = (mfma_ok && ni > kWaveCols) ? strips * chunks : 0;
         v32[kPfxStrip] = (mfma_ok && ni <= kWaveCols) ? strips : 0;
         v32[kPfxSplit] = (mfma_ok && ni > kWaveCols && ni <= kSplitCols) ? strips : 0;
@@ -190,7 +199,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         if (a.kind == 1) {
 #pragma unroll
             for (int q = 0; q < kNumPrefix; ++q)
-                if (q != kPfxRows) v32[q] = 0;
+                if (q >= kNumLists && q != kPfxRows) v32[q] = 0;
         }
         block_exclusive_scan<int32_t, kNumPrefix>(v32, t32, sScan32);
 
@@ -198,16 +207,12 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             SegRec rec;
             rec.off1 = o1; rec.off2 = o2; rec.offO = oO;
             rec.M = mi; rec.N = ni; rec.K = ki; rec.packLen = pack > 0 ? pack : 0;
-            rec.kind = strips == 0 ? kSegEmpty
-                       : !aligned ? kSegSlow
-                       : pack > 0 ? kSegPackLead
-                       : pack < 0 ? kSegPackFollow
-                       : ni <= kWaveCols ? kSegStrip
-                       : ni <= kSplitCols ? kSegSplit : kSegWide;
-            rec.pad_ = 0;
+            rec.kind = seg_kind;
+            rec.index = (int32_t)g;
             pv.recs[g] = rec;
 #pragma unroll
-            for (int q = 0; q < kNumPrefix; ++q) pv.pfx[q][g] = base32[q] + v32[q];
+            for (int q = 0; q < kNumLists; ++q)          // v32 now holds the exclusive scans
+                if (cls == q) pv.list[q][base32[q] + v32[q]] = rec;
             if (!offsets_given) {
                 if (a.a1) a.a1[g] = o1;
                 if (a.a2) a.a2[g] = o2;
@@ -220,7 +225,6 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             }
         }
         maxM = max(maxM, mi); maxN = max(maxN, ni); maxK = max(maxK, ki); nbad += bad ? 1 : 0;
-        nrest += (a.kind == 0 && mfma_ok && strips > 0 && ni <= kWaveCols && !fast_strip_shape(ni, ki)) ? 1 : 0;
 #pragma unroll
         for (int q = 0; q < kNumPrefix; ++q) base32[q] += t32[q];
         if (!offsets_given) {
@@ -235,8 +239,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     // wavefront, then thread 0 folds the 16 partial results.
     maxM = wave_max_nonneg(maxM); maxN = wave_max_nonneg(maxN); maxK = wave_max_nonneg(maxK);
     nbad = __builtin_amdgcn_readlane(wave_inclusive_scan(nbad), 63);
-    nrest = __builtin_amdgcn_readlane(wave_inclusive_scan(nrest), 63);
-    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; sRed[wave][4] = nrest; }
+    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; }
     __syncthreads();
 
     if (tid == 0) {
@@ -251,11 +254,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             if (a.a2) a.a2[nseg] = D2;
             if (a.aO) a.aO[nseg] = DO;
         }
-        int32_t rM = 0, rN = 0, rK = 0, rBad = 0, rRest = 0;
+        int32_t rM = 0, rN = 0, rK = 0, rBad = 0;
         for (int w = 0; w < kSchedWaves; ++w) {
-            rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3]; rRest += sRed[w][4];
+            rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3];
         }
-        for (int q = 0; q < kNumPrefix; ++q) pv.pfx[q][nseg] = base32[q];
         PlanHeader *h = pv.hdr;
         h->magic = kPlanMagic;
         h->nseg = (int32_t)nseg;
@@ -263,11 +265,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->kind = a.kind;
         h->Dm1 = D1; h->Dm2 = D2; h->Dout = DO;
         h->total_rows = base32[kPfxRows];
-        for (int q = 0; q < 8; ++q) h->totals[q] = q < kNumPrefix ? base32[q] : 0;
+        for (int q = 0; q < 12; ++q) h->totals[q] = q < kNumPrefix ? base32[q] : 0;
         h->max_M = rM; h->max_N = rN; h->max_K = rK;
         h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
         h->run_errors = 0;
-        h->strip_rest = rRest;
     }
 }
 

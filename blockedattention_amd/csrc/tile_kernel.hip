@@ -79,18 +79,21 @@ __global__ __launch_bounds__(kTileThreads, 2) void tile_kernel(RunArgs a, int zd
     const int pair = (slot / zdim) * kDies + die;
     const int z0 = slot % zdim;
     const int H = (int)a.H;
-    if (pair >= a.nseg * H) return;
-    const int g = pair % a.nseg;
-    const int64_t h = pair / a.nseg;
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     const bool ok = header_ok(a);
-    const Seg s = load_seg(pv, g, h, a);
-    const int kind = pv.recs[g].kind;
     if (!ok) {
         if (!(a.flags & kFlagQuiet) && blockIdx.x == 0 && threadIdx.x == 0)
             atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
     }
+    // pairs = (entries of the work list) x heads, entry fastest
+    const int entries = a.list < 0 ? a.nseg : (int)((ConstHdr)(uintptr_t)a.plan)->totals[a.list];
+    if (entries <= 0 || pair >= entries * H) return;
+    const int64_t h = pair / entries;
+    bool valid;
+    const Seg s = load_listed(pv, pair % entries, h, a, valid);
+    if (!valid) return;
+    const int kind = s.kind;
     if (!tile_segment(kind, s.N, s.K)) return;
     const int M = s.M, N = s.N, K = s.K;
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
@@ -365,15 +368,13 @@ static void launch_one(const RunArgs &args, unsigned groups, int zdim, hipStream
 
 // Launches the tile kernel over (segment, head, row block).  With a plan summary the row-block
 // dimension covers the tallest segment; without it the workgroups loop over row blocks.
-int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t nseg, const ba_plan_info *info,
+int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                  hipStream_t stream) {
     int64_t z = 4;
-    if (info) {
-        nseg = info->nseg;
+    if (info)
         z = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kTileRows - 1) / kTileRows));
-    }
-    if (nseg <= 0) return BA_OK;
-    const int64_t pairs = nseg * args.H;
+    if (slots <= 0) return BA_OK;
+    const int64_t pairs = slots * args.H;
     const int64_t groups = (pairs + kDies - 1) / kDies * kDies * z;
     if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
     const bool f32out = args.flags & kFlagOutF32;

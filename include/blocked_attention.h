@@ -65,7 +65,12 @@ typedef struct ba_plan_info {
     int32_t max_M, max_N, max_K;
     int32_t bad_segments;   /* segments rejected by the device-side checks */
     int32_t run_errors;     /* kernels that refused to run against this plan */
-    int32_t strip_rest;     /* strip-class segments too large for the strip kernel's LDS window */
+    /* segments per launch class (lengths of the plan's work lists) */
+    int32_t list_small;     /* strip kernel, main launch */
+    int32_t list_big;       /* strip kernel, second launch with the 64 KiB window */
+    int32_t list_tile;      /* tile kernel (large segments) */
+    int32_t list_rest;      /* segment kernel: packs, element-wise class, leftovers */
+    int32_t reserved;
 } ba_plan_info;
 
 const char *ba_status_string(int status);
