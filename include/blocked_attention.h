@@ -56,10 +56,11 @@ typedef struct ba_plan_info {
     int64_t nseg;
     int64_t Dm1, Dm2, Dout; /* last prefix-sum entries = elements per head */
     int64_t total_rows;     /* sum of M */
-    int64_t gemm_items;     /* 16 x <=256 output pieces of the GEMM-only kernel */
-    int64_t strip_items;    /* 16-row strips with N <= 256 (one wavefront each) */
-    int64_t split_items;    /* 16-row strips with 256 < N <= 4096 (one workgroup each) */
-    int64_t wide_items;     /* 16-row strips with N > 4096 (two-sweep path) */
+    /* work-item totals (16-row strips) by segment shape */
+    int64_t gemm_items;     /* 16 x <=256 output pieces of segments with N > 256 */
+    int64_t strip_items;    /* 16-row strips of aligned segments with N <= 256 */
+    int64_t split_items;    /* 16-row strips with 256 < N <= 4096 */
+    int64_t wide_items;     /* 16-row strips with N > 4096 */
     int64_t pack_items;     /* packs of tiny segments sharing one wavefront */
     int64_t slow_items;     /* 16-row strips of segments that need the element-wise path */
     int32_t max_M, max_N, max_K;
@@ -88,7 +89,7 @@ size_t ba_plan_bytes(int64_t nseg);
  * __getTiling (csrc/cuda/spBlkGEMM.cu:943-983): one kernel, no host round
  * trip.  Depending on `mode` it reads or writes MList/NList/KList (int64[nseg])
  * and accum1/accum2/accumOut (int64[nseg+1]); the plan receives offsets, sizes
- * and the scanned work-item counts every compute kernel searches.
+ * and one compacted work list per compute-kernel launch.
  * In BA_META_FROM_ACCUM the lists are derived in exact integer arithmetic.
  * Output pointers may be NULL when the caller does not need that half.
  */
