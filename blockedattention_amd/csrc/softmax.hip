@@ -135,7 +135,7 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
         const int r0 = 16 * strip + rg;
         f32x4 x[G];
 #pragma unroll
-        for (int g = 0; g < G; ++g) x[g] = f32x4{-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
+        for (int g = 0; g < G; ++g) x[g] = f32x4{-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f} * sgn;   // lowest after the sign flip
         if (!BACKWARD) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)

@@ -73,3 +73,33 @@ def test_config5_full_size_properties(dev):
         assert ((got - ref).abs() <= 1e-3 + ref * 2.0 ** -8).all(), (g, h, r)
         assert ((got - ref.bfloat16().float()).abs() <= ref * 2.0 ** -7 + 1e-9).all(), (g, h, r)
     assert plan.read().run_errors == 0
+
+
+def test_long_k_and_every_launch_class(dev):
+    # K > 128 (A fragments reloaded per 128-k span in the tile kernel, K slabs in the segment kernel),
+    # ragged K, and one call that exercises all four work lists at once.
+    M = [40, 130, 20, 64, 7, 5, 300, 33]; N = [48, 300, 200, 256, 6, 9, 129, 64]; K = [160, 256, 200, 128, 16, 16, 136, 264]
+    for dtype, scale in ((torch.float16, 0.05), (torch.bfloat16, -0.05)):
+        plan = run_all(dev, M, N, K, 2, dtype, scale, seed=3)
+        i = plan.info
+        # (64,256,128): 16 tiles x 4 k-steps = 64 blocks -> big; (7,6,16)+(5,9,16) pack; N >= 128 with long K -> tile
+        assert i.list_big == 1 and i.list_tile == 3 and i.list_small == 0
+        assert i.list_small + i.list_big + i.list_tile + i.list_rest + 1 == len(M)      # one pack follower
+
+
+def test_work_lists_match_the_shape_rules(dev):
+    # The lengths of the four work lists against the classification restated on the host.
+    for cfg in (1, 2, 3, 4, 5):
+        w = workloads.make(cfg)
+        plan = make_plan(dev, w.M, w.N, w.K)
+        i = plan.info
+        tiles = 2 * ((w.N + 31) // 32); nks = (w.K + 31) // 32
+        blocks = np.where((w.N >= 2) & (w.N <= 256) & (nks >= 1) & (nks <= 4), tiles * nks, 0)
+        aligned = (w.K % 8 == 0)                       # offsets of these configurations are multiples of 8 with K
+        packed = i.list_small + i.list_big + i.list_tile + i.list_rest
+        small = int(((blocks >= 1) & (blocks <= 32) & aligned).sum())
+        big = int(((blocks > 32) & (blocks <= 64) & aligned).sum())
+        assert i.list_big == big, cfg
+        assert i.list_small <= small and small - i.list_small <= 2 * i.pack_items * 8, cfg   # packs take tiny ones
+        assert i.list_tile == int(((w.N > 256) | ((w.N >= 128) & (blocks == 0))).sum()), cfg
+        assert packed <= w.nseg
