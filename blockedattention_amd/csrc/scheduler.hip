@@ -141,7 +141,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         // consecutive tiny aligned segments (same K, sum M <= 16, sum N <= 16).
         // The first lane of every window walks its 16 entries in registers.
         int32_t pack = 0;
-        if (a.kind == 0) {
+        // Only batches that contain segments small enough to pack pay for the window walk.
+        const bool packable = aligned && mi >= 1 && ni >= 1 && ki >= 1 && mi < kPackDim && ni < kPackDim;
+        if (a.kind == 0 && __syncthreads_or(packable)) {
             sM[tid] = mi; sN[tid] = ni; sK[tid] = aligned ? ki : -1; sPack[tid] = 0;
             __syncthreads();
             if ((tid & 15) == 0) {
@@ -155,7 +157,17 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
                     wn[j] = vn.x; wn[j + 1] = vn.y; wn[j + 2] = vn.z; wn[j + 3] = vn.w;
                     wk[j] = vk.x; wk[j + 1] = vk.y; wk[j + 2] = vk.z; wk[j + 3] = vk.w;
                 }
+                // follow: bit j = entry j joins the pack before it; lens: 5 bits per entry = pack length at
+                // its leader.  Both stay in registers; the window's lanes decode them after the barrier.
+                uint32_t follow = 0;
+                uint64_t lens_lo = 0, lens_hi = 0;              // entries 0..11 / 12..15
                 int start = 0, len = 0, sumM = 0, sumN = 0, kcur = 0;
+                auto close = [&]() {
+                    if (len >= 2) {
+                        if (start < 12) lens_lo |= (uint64_t)len << (5 * start);
+                        else lens_hi |= (uint64_t)len << (5 * (start - 12));
+                    }
+                };
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
                     const bool ok = wm[j] >= 1 && wn[j] >= 1 && wk[j] >= 1;
@@ -163,16 +175,27 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
                                       sumN + wn[j] <= kPackDim;
                     if (fits) {
                         sumM += wm[j]; sumN += wn[j]; ++len;
-                        sPack[tid + j] = -1;
+                        follow |= 1u << j;
                     } else {
-                        if (len >= 2) sPack[tid + start] = len;
+                        close();
                         start = j; len = ok ? 1 : 0; sumM = wm[j]; sumN = wn[j]; kcur = wk[j];
                     }
                 }
-                if (len >= 2) sPack[tid + start] = len;
+                close();
+                sPack[tid] = (int32_t)follow;
+                sPack[tid + 1] = (int32_t)(uint32_t)lens_lo;
+                sPack[tid + 2] = (int32_t)(uint32_t)(lens_lo >> 32);
+                sPack[tid + 3] = (int32_t)(uint32_t)lens_hi;
             }
             __syncthreads();
-            pack = sPack[tid];
+            {
+                const int wbase = tid & ~15, j = tid & 15;
+                const uint32_t follow = (uint32_t)sPack[wbase];
+                const uint64_t lens_lo = (uint32_t)sPack[wbase + 1] | ((uint64_t)(uint32_t)sPack[wbase + 2] << 32);
+                const uint64_t lens_hi = (uint32_t)sPack[wbase + 3];
+                const int len = (int)((j < 12 ? lens_lo >> (5 * j) : lens_hi >> (5 * (j - 12))) & 31);
+                pack = ((follow >> j) & 1) ? -1 : len;
+            }
         }
 
         const int32_t strips = (ni >= 1) ? (mi + kStripRows - 1) / kStripRows : 0;
