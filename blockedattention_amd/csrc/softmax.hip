@@ -309,6 +309,7 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
                     }
                 }
                 sum = wave_sum(sum);
+                if (c == 0.f) sum = (float)cols;           // scale 0: the padding slots counted as exp2(0) too
                 const float inv = __builtin_amdgcn_rcpf(sum);
 #pragma unroll
                 for (int k = 0; k < kRowSteps; ++k) {

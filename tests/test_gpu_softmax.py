@@ -46,7 +46,7 @@ def test_long_rows_127x2047_half(dev):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_mixed_widths_scale_and_no_column_limit(dev, dtype):
     rows = [3, 5, 0, 2, 4, 1]; cols = [1, 63, 12, 1025, 9000, 64]       # 9000 > the reference's 8191 limit
-    for scale in (1.0, 0.125, -0.7):
+    for scale in (1.0, 0.125, -0.7, 0.0):
         src, out, _ = run_softmax(dev, rows, cols, 2, dtype, scale=scale, seed=4)
         assert_probs_close(out, oracle.per_segment_torch_softmax(src, rows, cols, scale), f"scale {scale}")
 
