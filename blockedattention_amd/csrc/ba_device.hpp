@@ -74,16 +74,31 @@ __device__ __forceinline__ float quad_column_sum(float v) {
     return v;
 }
 
-// Full-wave reductions (all 64 lanes end with the result).
+// Full-wave reductions (all 64 lanes end with the result): data-parallel-primitive row shifts and row
+// broadcasts accumulate into lane 63, which is then read back as a scalar.  No LDS round trips.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_or(float v, float identity) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity),
+                                                                 __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf,
+                                                                 false));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
+    const float lowest = -INFINITY;
+    v = fmaxf(v, dpp_or<0x111, 0xf>(v, lowest));   // row_shr:1
+    v = fmaxf(v, dpp_or<0x112, 0xf>(v, lowest));   // row_shr:2
+    v = fmaxf(v, dpp_or<0x114, 0xf>(v, lowest));   // row_shr:4
+    v = fmaxf(v, dpp_or<0x118, 0xf>(v, lowest));   // row_shr:8
+    v = fmaxf(v, dpp_or<0x142, 0xa>(v, lowest));   // row_bcast:15 into rows 1 and 3
+    v = fmaxf(v, dpp_or<0x143, 0xc>(v, lowest));   // row_bcast:31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
+    v += dpp_or<0x111, 0xf>(v, 0.f);
+    v += dpp_or<0x112, 0xf>(v, 0.f);
+    v += dpp_or<0x114, 0xf>(v, 0.f);
+    v += dpp_or<0x118, 0xf>(v, 0.f);
+    v += dpp_or<0x142, 0xa>(v, 0.f);
+    v += dpp_or<0x143, 0xc>(v, 0.f);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // Values that are the same in every lane of the wavefront by construction

@@ -78,7 +78,8 @@ struct PlanHeader {
     int32_t max_M, max_N, max_K;
     int32_t bad_segments;
     int32_t run_errors;      // bumped by kernels that refuse to run
-    int32_t pad_[23];
+    int32_t small_max_N, small_max_M;   // maxima over the segments of the strip kernel's main launch
+    int32_t pad_[21];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 

@@ -753,9 +753,9 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     const int64_t n_rest = !mfma_ok ? nseg : info ? info->list_rest : nseg;
     const bool lean = info && info->max_N <= 128;
     // z: enough workgroups to fill the machine, at most one per kSegWaves strips of the tallest segment
-    auto strip_z = [&](int64_t slots) {
+    auto strip_z = [&](int64_t slots, int64_t tallest) {
         if (!info) return (int64_t)2;
-        const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(info->max_M, 1), kStripRows), kSegWaves);
+        const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(tallest, 1), kStripRows), kSegWaves);
         const int64_t want = ceil_div((int64_t)cus * 8, std::max<int64_t>(1, slots * (int64_t)H));
         return std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
     };
@@ -765,14 +765,18 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
         RunArgs fa = args;
         fa.list = pass == 0 ? kListSmall : kListBig;
         fa.lds_blocks = pass == 0 ? kFastBlocks : kBigBlocks;
+        bool lean_pass = lean;
         if (info && pass == 0) {
-            const int64_t nt = fast_strip_tiles((int)std::min<int64_t>(std::max<int64_t>(info->max_N, 1), kWaveCols));
+            // the main launch is sized by ITS widest and tallest segment, not the batch's
+            const int64_t nt = fast_strip_tiles((int)std::max(info->small_max_N, 1));
             const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
             fa.lds_blocks = (int)std::min<int64_t>(kFastBlocks, nt * nks);
+            lean_pass = info->small_max_N <= 128;
         }
-        const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots));
+        const int64_t tallest = !info ? 0 : pass == 0 ? info->small_max_M : info->max_M;
+        const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots, tallest));
         const size_t lds_bytes = (size_t)fa.lds_blocks * kLdsBlockBytes;
-        if (lean)
+        if (lean_pass)
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         else
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream, fa);

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
     __shared__ __attribute__((aligned(16))) int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads];
     __shared__ int32_t sPack[kSchedThreads];
-    __shared__ int32_t sRed[kSchedWaves][4];
+    __shared__ int32_t sRed[kSchedWaves][6];
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6), lane = lane_id();
@@ -98,6 +98,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     int64_t base64[3] = {0, 0, 0};
     int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
+    int32_t maxSmallN = 0, maxSmallM = 0;       // widest / tallest segment of the strip kernel's main launch
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
 
     for (int64_t chunk = 0; chunk < nseg || chunk == 0; chunk += kSchedThreads) {
@@ -248,6 +249,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             }
         }
         maxM = max(maxM, mi); maxN = max(maxN, ni); maxK = max(maxK, ki); nbad += bad ? 1 : 0;
+        if (cls == kListSmall) { maxSmallN = max(maxSmallN, ni); maxSmallM = max(maxSmallM, mi); }
 #pragma unroll
         for (int q = 0; q < kNumPrefix; ++q) base32[q] += t32[q];
         if (!offsets_given) {
@@ -261,8 +263,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     // Shape maxima and the count of rejected segments: DPP reduction per
     // wavefront, then thread 0 folds the 16 partial results.
     maxM = wave_max_nonneg(maxM); maxN = wave_max_nonneg(maxN); maxK = wave_max_nonneg(maxK);
+    maxSmallN = wave_max_nonneg(maxSmallN); maxSmallM = wave_max_nonneg(maxSmallM);
     nbad = __builtin_amdgcn_readlane(wave_inclusive_scan(nbad), 63);
-    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; }
+    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; sRed[wave][4] = maxSmallN; sRed[wave][5] = maxSmallM; }
     __syncthreads();
 
     if (tid == 0) {
@@ -277,9 +280,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             if (a.a2) a.a2[nseg] = D2;
             if (a.aO) a.aO[nseg] = DO;
         }
-        int32_t rM = 0, rN = 0, rK = 0, rBad = 0;
+        int32_t rM = 0, rN = 0, rK = 0, rBad = 0, rSN = 0, rSM = 0;
         for (int w = 0; w < kSchedWaves; ++w) {
             rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3];
+            rSN = max(rSN, sRed[w][4]); rSM = max(rSM, sRed[w][5]);
         }
         PlanHeader *h = pv.hdr;
         h->magic = kPlanMagic;
@@ -290,6 +294,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->total_rows = base32[kPfxRows];
         for (int q = 0; q < 12; ++q) h->totals[q] = q < kNumPrefix ? base32[q] : 0;
         h->max_M = rM; h->max_N = rN; h->max_K = rK;
+        h->small_max_N = rSN; h->small_max_M = rSM;
         h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
         h->run_errors = 0;
     }

@@ -71,6 +71,8 @@ typedef struct ba_plan_info {
     int32_t list_big;       /* strip kernel, second launch with the 64 KiB window */
     int32_t list_tile;      /* tile kernel (large segments) */
     int32_t list_rest;      /* segment kernel: packs, element-wise class, leftovers */
+    int32_t small_max_N;    /* widest segment of the strip kernel's main launch */
+    int32_t small_max_M;    /* tallest segment of the strip kernel's main launch */
     int32_t reserved;
 } ba_plan_info;
 
