@@ -1,31 +1,28 @@
 // Varlen GEMM (S_g = A_g B_g^T) and the fused GEMM + row softmax for fp16/bf16
 // on gfx950: MFMA 16x16x32 with fp32 accumulation, scores kept in registers.
+// This file holds the two kernels for segments of up to 256 columns and the
+// launcher of a whole call; large segments are tile_kernel.hip.
 //
-// Work decomposition (all counts come scanned from the plan):
-//   pack item   one wavefront, several tiny segments sharing one 16x16 MFMA tile
-//   strip item  one wavefront, 16 rows x all N <= 256 columns of one segment
-//   gemm item   one wavefront, 16 rows x one 256-column chunk (GEMM only, any N)
-//   split item  one 16-wave workgroup, 16 rows x all 256 < N <= 4096 columns
-//   wide item   one workgroup, 16 rows x N > 4096 columns in two sweeps
-//
-// The MFMA is issued "transposed": the B_g rows go in as the first operand and
-// the A_g rows as the second, so that a lane ends up with four CONSECUTIVE
-// columns of ONE score row (row = lane%16, columns 4*(lane/16)+i of each
-// 16-wide tile).  Row maxima and sums are then in-lane loops plus two
-// cross-lane steps, and stores are 8-byte runs along the row.
+//   strip_kernel    strip-class segments whose B_g fits an LDS window: B_g is
+//                   copied to LDS once per workgroup, each wavefront computes
+//                   16-row strips with code specialised for the exact tile count
+//                   and with lane order following memory order (strips_exact).
+//   segment_kernel  everything that needs care instead of speed: packs of tiny
+//                   segments sharing one MFMA tile (wave_pack), segments that
+//                   break the 16-byte operand alignment (K % 8 != 0, odd segment
+//                   starts, transposed layouts: element-wise generic_rows),
+//                   strip-class leftovers whose B_g is walked in K slabs
+//                   (strips_from_lds).
 //
 // Both operands are K-contiguous (A_g is M x K, B_g is N x K), so a lane's
-// eight k-values are one 16-byte global load straight into the MFMA operand
-// registers; no transposition is ever needed.  Segments that break the
-// alignment this needs (K % 8 != 0, odd segment starts, transposed layouts)
-// take an element-wise loader into the same MFMA code.
+// eight k-values are one 16-byte load straight into an MFMA operand register;
+// no transposition is ever needed.
 #include <algorithm>
 
 #include "ba_gemm_common.hpp"
 
 namespace ba {
 
-constexpr int kGroupThreads = 64 * kWavesPerGroup;
 constexpr int kMaxTiles = kWaveCols / 16;  // 16 MFMA tiles per wavefront
 
 // ------------------------------------------------------------ operand loads
@@ -89,51 +86,6 @@ __device__ __attribute__((noinline)) void generic_rows(const uint16_t *aseg, con
                               __builtin_amdgcn_exp2f(
                                   fmaf(sgn * generic_dot<DT>(aseg, bseg, r, col, M, N, K, t1, t2), c, bias)) * inv,
                               f32out);
-        }
-    }
-}
-
-// ------------------------------------------------------------------- scores
-// acc[t] (t < NT) <- rows r0..r0+15 x columns c0+16t..c0+16t+15 of A_g B_g^T, for
-// segments whose operand rows are 16-byte aligned.
-// Rows and columns past the segment read as zeros (buffer range check); the
-// callers discard those results.
-template <int DT, int NT>
-__device__ __forceinline__ void stage_scores(f32x4 (&acc)[kMaxTiles], const Seg &s, const SegRes &res, int r0,
-                                             int c0) {
-    const int lane = lane_id(), l16 = lane & 15, q = lane >> 4;
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const int K = s.K;
-    // One lane offset serves A and B alike: row l16 of the tile, k-group q.
-    const int voff = (l16 * K + q * 8) * 2;
-    const int a_soff = r0 * K * 2;
-    // Loads are issued in batches of at most kBatch tiles so that the operand
-    // registers in flight stay well below the accumulator count.
-    constexpr int kBatch = NT < 4 ? NT : 4;
-    const int kfull = K & ~31;
-    for (int k0 = 0; k0 < kfull; k0 += 32) {
-        const u32x4 af = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + k0 * 2, 0);
-#pragma unroll
-        for (int tb = 0; tb < NT; tb += kBatch) {
-            u32x4 bf[kBatch];
-#pragma unroll
-            for (int t = 0; t < kBatch; ++t)
-                bf[t] = __builtin_amdgcn_raw_buffer_load_b128(res.b, voff, ((c0 + (tb + t) * 16) * K + k0) * 2, 0);
-#pragma unroll
-            for (int t = 0; t < kBatch; ++t) acc[tb + t] = Elem<DT>::mfma(bf[t], af, acc[tb + t]);
-        }
-    }
-    if (kfull < K) {   // K % 32 in {8, 16, 24}: lanes whose k-group lies past K feed zeros
-        const bool live = kfull + q * 8 < K;
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        u32x4 af = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff, a_soff + kfull * 2, 0);
-        af = live ? af : zero;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            u32x4 bf = __builtin_amdgcn_raw_buffer_load_b128(res.b, voff, ((c0 + t * 16) * K + kfull) * 2, 0);
-            bf = live ? bf : zero;
-            acc[t] = Elem<DT>::mfma(bf, af, acc[t]);
         }
     }
 }
@@ -251,32 +203,6 @@ __device__ __forceinline__ void store_rows(const f32x4 (&acc)[kMaxTiles], int nt
 }
 
 
-// One wavefront, one strip, everything in registers.
-template <int DT, int NT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void wave_strip(int nt, const Seg &s, const RunArgs &a, int r0, int c0) {
-    f32x4 acc[kMaxTiles];
-    const SegRes res = make_res(s, a.A, a.B);
-    stage_scores<DT, NT>(acc, s, res, r0, c0);
-    float factor = 1.f;
-    if (FUSED) {
-        float c = a.scale * kLog2e;
-        prepare_scores<NT>(acc, nt, s.N, c0, c);
-        float m, l;
-        local_softmax<NT>(acc, nt, c, m, l);
-        factor = 1.f / l;
-    }
-    store_rows<DT, NT, F32OUT>(acc, nt, s, a.out, r0, c0, factor);
-}
-
-template <int DT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void wave_strip_dispatch(int nt, const Seg &s, const RunArgs &a, int r0, int c0) {
-    if (nt <= 1) wave_strip<DT, 1, FUSED, F32OUT>(nt, s, a, r0, c0);
-    else if (nt <= 2) wave_strip<DT, 2, FUSED, F32OUT>(nt, s, a, r0, c0);
-    else if (nt <= 4) wave_strip<DT, 4, FUSED, F32OUT>(nt, s, a, r0, c0);
-    else if (nt <= 8) wave_strip<DT, 8, FUSED, F32OUT>(nt, s, a, r0, c0);
-    else wave_strip<DT, 16, FUSED, F32OUT>(nt, s, a, r0, c0);
-}
-
 template <int DT, bool FUSED>
 __device__ __forceinline__ void generic_seg_rows(const Seg &s, const RunArgs &a, int r_begin, int r_end,
                                                  int c_begin, int c_end) {
@@ -354,30 +280,6 @@ __device__ __forceinline__ void wave_pack(const PlanRO &pv, int g, int len, int6
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         if (keep[i]) store_one<DT>(a.out, e0 + cLoc[i], v[i], F32OUT);
-}
-
-// Combines the per-wavefront (maximum, sum) pairs of one strip through LDS.
-// Returns the factor this wavefront's exp2((s - m_wave) * c) values must be
-// multiplied by; gshift receives the subtracted global maximum and ginv 1/sum.
-__device__ __forceinline__ float exchange_row_stats(float (*sM)[16], float (*sL)[16], int wave, float m, float l,
-                                                    float c, float &gshift, float &ginv) {
-    const int lane = lane_id(), l16 = lane & 15;
-    if (lane < 16) { sM[wave][l16] = m; sL[wave][l16] = l; }
-    __syncthreads();
-    float gm = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < kWavesPerGroup; ++w) gm = fmaxf(gm, sM[w][l16]);
-    gshift = (gm == -INFINITY) ? 0.f : gm;
-    float gl = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWavesPerGroup; ++w) {
-        const float mw = sM[w][l16];
-        const float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mw - gshift) * c);
-        gl += sL[w][l16] * f;
-    }
-    ginv = 1.f / gl;
-    const float mine = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m - gshift) * c);
-    return mine * ginv;
 }
 
 // ------------------------------------------------------ LDS-staged strips

@@ -179,8 +179,10 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
 
 // grid (segment, head, z): the wavefronts of the workgroups with the same (segment, head) share the
 // segment's 16-row strips round-robin.
-template <int DT, bool BACKWARD>
-__global__ __launch_bounds__(kSoftmaxThreads) void softmax_runs_kernel(SoftmaxArgs a) {
+// MAXG = 8 is the build for batches whose widest row has 128 columns or fewer: half the registers,
+// twice the resident wavefronts.
+template <int DT, bool BACKWARD, int MAXG>
+__global__ __launch_bounds__(kSoftmaxThreads, MAXG <= 8 ? 3 : 1) void softmax_runs_kernel(SoftmaxArgs a) {
     typedef typename Io<DT>::T T;
     const int nseg = softmax_plan_nseg(a);
     const int g = blockIdx.x;
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_runs_kernel(SoftmaxAr
     const PlanRO pv = plan_ro(a.plan, nseg);
     const SegRec rec = load_rec(pv.recs, g);
     const int rows = rec.M, cols = rec.N;
-    if (cols < 1 || cols > kRunCols || rows < 1) return;
+    if (cols < 1 || cols > kRunCols || cols > 16 * MAXG || rows < 1) return;
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int first = blockIdx.z * kSoftmaxWaves + wave, step = gridDim.z * kSoftmaxWaves;
     const int64_t seg0 = (int64_t)blockIdx.y * a.Dsrc + rec.offO;
@@ -211,8 +213,15 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_runs_kernel(SoftmaxAr
     const int tiles = fast_strip_tiles(cols);
 #define BA_RUNS(G_) case G_: softmax_runs<DT, G_, BACKWARD>(a, seg0, rows, cols, first, step); break;
     switch (tiles) {
-        BA_RUNS(2) BA_RUNS(4) BA_RUNS(6) BA_RUNS(8) BA_RUNS(10) BA_RUNS(12) BA_RUNS(14) BA_RUNS(16)
-        default: break;
+        BA_RUNS(2) BA_RUNS(4) BA_RUNS(6) BA_RUNS(8)
+        default:
+            if (MAXG > 8) {
+                switch (tiles) {
+                    BA_RUNS(10) BA_RUNS(12) BA_RUNS(14) BA_RUNS(16)
+                    default: break;
+                }
+            }
+            break;
     }
 #undef BA_RUNS
 }
@@ -376,8 +385,11 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
         z_rows = std::max<int64_t>(1, std::min<int64_t>(4 * want, (info->max_M + kSoftmaxWaves - 1) / kSoftmaxWaves));
     }
     if (nseg <= 0) return BA_OK;
-    hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD>), dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs),
-                       dim3(kSoftmaxThreads), 0, stream, args);
+    const dim3 grid_runs((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs);
+    if (info && info->max_N <= 128)
+        hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 8>), grid_runs, dim3(kSoftmaxThreads), 0, stream, args);
+    else
+        hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 16>), grid_runs, dim3(kSoftmaxThreads), 0, stream, args);
     if (rows_work)
         hipLaunchKernelGGL((softmax_rows_kernel<DT, BACKWARD>),
                            dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z_rows), dim3(kSoftmaxThreads), 0, stream,
