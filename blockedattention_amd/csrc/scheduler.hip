@@ -16,8 +16,7 @@ __device__ __forceinline__ int64_t readlane_t(int64_t v, int l) {
     return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-constexpr int kSchedThreads = 1024;
-constexpr int kSchedWaves = kSchedThreads / 64;
+constexpr int kSchedThreadsMax = 1024;   // one workgroup; batches of up to 256 segments use a 256-thread build
 
 struct SchedArgs {
     void *plan;
@@ -32,7 +31,7 @@ struct SchedArgs {
 // scans, then the 16 wavefront totals are scanned by lanes 0..15 of every
 // wavefront (one row of DPP shifts).  lds holds NQ * kSchedWaves entries and
 // is free for reuse after the next __syncthreads().  One barrier.
-template <typename T, int NQ>
+template <typename T, int NQ, int kSchedWaves>
 __device__ __forceinline__ void block_exclusive_scan(T (&v)[NQ], T (&total)[NQ], T *lds) {
     const int wave = uniform((int)(threadIdx.x >> 6)), lane = lane_id();
     T incl[NQ];
@@ -83,7 +82,9 @@ __device__ __forceinline__ bool derive_lists(int64_t mk, int64_t nk, int64_t mn,
     return n * k == nk;
 }
 
+template <int kSchedThreads>
 __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
+    constexpr int kSchedWaves = kSchedThreads / 64;
     __shared__ int64_t sScan64[kSchedWaves * 3];
     __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
     __shared__ __attribute__((aligned(16))) int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads];
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         // Offsets first: alignment decides which path a segment takes.
         int64_t v64[3] = {m * k, n * k, m * n}, t64[3] = {0, 0, 0};
         if (!offsets_given) {
-            block_exclusive_scan<int64_t, 3>(v64, t64, sScan64);
+            block_exclusive_scan<int64_t, 3, kSchedWaves>(v64, t64, sScan64);
             o1 = base64[0] + v64[0]; o2 = base64[1] + v64[1]; oO = base64[2] + v64[2];
         }
         // 16-byte operand rows, and segment areas that fit the 32-bit byte
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             for (int q = 0; q < kNumPrefix; ++q)
                 if (q >= kNumLists && q != kPfxRows) v32[q] = 0;
         }
-        block_exclusive_scan<int32_t, kNumPrefix>(v32, t32, sScan32);
+        block_exclusive_scan<int32_t, kNumPrefix, kSchedWaves>(v32, t32, sScan32);
 
         if (live) {
             SegRec rec;
@@ -314,7 +315,8 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
         return BA_ERR_INVALID_ARG;
     }
     SchedArgs args{plan, nseg, mode, kind, M, N, K, a1, a2, aO};
-    hipLaunchKernelGGL(schedule_kernel, dim3(1), dim3(kSchedThreads), 0, stream, args);
+    if (nseg <= 256) hipLaunchKernelGGL(schedule_kernel<256>, dim3(1), dim3(256), 0, stream, args);
+    else hipLaunchKernelGGL(schedule_kernel<kSchedThreadsMax>, dim3(1), dim3(kSchedThreadsMax), 0, stream, args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
