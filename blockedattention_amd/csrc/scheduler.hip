@@ -315,7 +315,8 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
         return BA_ERR_INVALID_ARG;
     }
     SchedArgs args{plan, nseg, mode, kind, M, N, K, a1, a2, aO};
-    if (nseg <= 256) hipLaunchKernelGGL(schedule_kernel<256>, dim3(1), dim3(256), 0, stream, args);
+    if (nseg <= 64) hipLaunchKernelGGL(schedule_kernel<64>, dim3(1), dim3(64), 0, stream, args);
+    else if (nseg <= 256) hipLaunchKernelGGL(schedule_kernel<256>, dim3(1), dim3(256), 0, stream, args);
     else hipLaunchKernelGGL(schedule_kernel<kSchedThreadsMax>, dim3(1), dim3(kSchedThreadsMax), 0, stream, args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
