@@ -86,12 +86,17 @@ __global__ __launch_bounds__(kTileThreads, 2) void tile_kernel(RunArgs a, int zd
             atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
     }
-    // pairs = (entries of the work list) x heads, entry fastest
+    // pairs = (entries of the work list, padded to a multiple of the die count) x heads, entry fastest,
+    // and the entries rotated by the head: die d works on entries = (d + h) mod 8 of head h, so over the
+    // heads every die sees every segment about equally often, however unequal the segments are.
     const int entries = a.list < 0 ? a.nseg : (int)((ConstHdr)(uintptr_t)a.plan)->totals[a.list];
-    if (entries <= 0 || pair >= entries * H) return;
-    const int64_t h = pair / entries;
+    const int padded = (entries + kDies - 1) / kDies * kDies;
+    if (entries <= 0 || pair >= padded * H) return;
+    const int h = pair / padded;
+    const int entry = (pair % padded + h) % padded;
+    if (entry >= entries) return;
     bool valid;
-    const Seg s = load_listed(pv, pair % entries, h, a, valid);
+    const Seg s = load_listed(pv, entry, h, a, valid);
     if (!valid) return;
     const int kind = s.kind;
     if (!tile_segment(kind, s.N, s.K)) return;
@@ -374,8 +379,8 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
     if (info)
         z = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kTileRows - 1) / kTileRows));
     if (slots <= 0) return BA_OK;
-    const int64_t pairs = slots * args.H;
-    const int64_t groups = (pairs + kDies - 1) / kDies * kDies * z;
+    const int64_t pairs = (slots + kDies - 1) / kDies * kDies * args.H;   // entries padded to whole dies
+    const int64_t groups = pairs * z;
     if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
     const bool f32out = args.flags & kFlagOutF32;
     if (dtype == BA_F16) {
