@@ -41,24 +41,27 @@ __host__ __device__ inline bool fast_strip_shape(int N, int K) {
     return b >= 1 && b <= kBigBlocks;
 }
 
-// What the scheduler scans per segment.  The first four are 0/1 class flags whose
+// What the scheduler scans per segment.  The first five are 0/1 class flags whose
 // scan compacts the segment indices into one work list per launch (the arrays of
 // the plan hold those lists); the others are work-item counts of which only the
 // totals are kept (plan summary).
+constexpr int kRunCols = 256;     // widest row of the softmax lane-run kernel; wider rows take the row kernel
+
 enum PrefixKind {
     kListSmall = 0,  // strip-class segments for the strip kernel's main launch (<= kFastBlocks LDS blocks)
     kListBig = 1,    // strip-class segments for its second launch (<= kBigBlocks)
     kListTile = 2,   // segments of the tile kernel
     kListRest = 3,   // everything else that has work: pack leaders, element-wise class, leftovers
-    kNumLists = 4,
-    kPfxGemm = 4,   // GEMM only, N > 256: ceil(M/16) * ceil(N/256) per segment
-    kPfxStrip = 5,  // fused, N <= 256 and not packed: ceil(M/16)
-    kPfxSplit = 6,  // fused, 256 < N <= 4096: ceil(M/16)
-    kPfxWide = 7,   // fused, N > 4096: ceil(M/16)
-    kPfxRows = 8,   // softmax: M rows
-    kPfxPack = 9,   // 1 for the first segment of a pack of tiny segments, else 0
-    kPfxSlow = 10,  // ceil(M/16) for segments the 16-byte operand loads cannot serve
-    kNumPrefix = 11
+    kListRows = 4,   // segments of the softmax row kernel: N > kRunCols, any plan kind (independent of the four above)
+    kNumLists = 5,
+    kPfxGemm = 5,   // GEMM only, N > 256: ceil(M/16) * ceil(N/256) per segment
+    kPfxStrip = 6,  // fused, N <= 256 and not packed: ceil(M/16)
+    kPfxSplit = 7,  // fused, 256 < N <= 4096: ceil(M/16)
+    kPfxWide = 8,   // fused, N > 4096: ceil(M/16)
+    kPfxRows = 9,   // softmax: M rows
+    kPfxPack = 10,  // 1 for the first segment of a pack of tiny segments, else 0
+    kPfxSlow = 11,  // ceil(M/16) for segments the 16-byte operand loads cannot serve
+    kNumPrefix = 12
 };
 
 // A segment is "aligned" when K % 8 == 0 and its A and B offsets are multiples

@@ -97,6 +97,7 @@ __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_pla
     info->list_big = (int32_t)h.totals[kListBig];
     info->list_tile = (int32_t)h.totals[kListTile];
     info->list_rest = (int32_t)h.totals[kListRest];
+    info->list_rows = (int32_t)h.totals[kListRows];
     info->small_max_N = h.small_max_N;
     info->small_max_M = h.small_max_M;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     PlanView pv = plan_view(a.plan, nseg);
 
     int64_t base64[3] = {0, 0, 0};
-    int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
     int32_t maxSmallN = 0, maxSmallM = 0;       // widest / tallest segment of the strip kernel's main launch
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
@@ -214,6 +214,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         int32_t v32[kNumPrefix], t32[kNumPrefix];
 #pragma unroll
         for (int q = 0; q < kNumLists; ++q) v32[q] = cls == q ? 1 : 0;
+        const bool wide_rows = mi >= 1 && ni > kRunCols;      // the softmax row kernel's, whatever the plan kind
+        v32[kListRows] = wide_rows ? 1 : 0;
         v32[kPfxGemm] = (mfma_ok && ni > kWaveCols) ? strips * chunks : 0;
         v32[kPfxStrip] = (mfma_ok && ni <= kWaveCols) ? strips : 0;
         v32[kPfxSplit] = (mfma_ok && ni > kWaveCols && ni <= kSplitCols) ? strips : 0;
@@ -238,6 +240,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
 #pragma unroll
             for (int q = 0; q < kNumLists; ++q)          // v32 now holds the exclusive scans
                 if (cls == q) pv.list[q][base32[q] + v32[q]] = rec;
+            if (wide_rows) pv.list[kListRows][base32[kListRows] + v32[kListRows]] = rec;
             if (!offsets_given) {
                 if (a.a1) a.a1[g] = o1;
                 if (a.a2) a.a2[g] = o2;

@@ -28,7 +28,6 @@ namespace ba {
 constexpr int kSoftmaxThreads = 256;
 constexpr int kSoftmaxWaves = kSoftmaxThreads / 64;
 constexpr int kRowSteps = 8;      // 512-column steps a row keeps in registers (4096 columns)
-constexpr int kRunCols = 256;     // widest row of the lane-run kernel
 
 template <int DT> struct Io;
 template <> struct Io<BA_F16> {
@@ -268,11 +267,14 @@ __device__ __forceinline__ void store_eight(typename Io<DT>::T *p, int valid, co
 template <int DT, bool BACKWARD>
 __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxArgs a) {
     typedef typename Io<DT>::T T;
+    // walks the plan's list of wide segments: the grid is as long as the list (or longer, without a host
+    // copy of the plan summary)
     const int nseg = softmax_plan_nseg(a);
-    const int g = blockIdx.x;
-    if (g >= nseg) return;
+    if (nseg < 0) return;
+    const int count = (int)((ConstHdr)(uintptr_t)a.plan)->totals[kListRows];
     const PlanRO pv = plan_ro(a.plan, nseg);
-    const SegRec rec = load_rec(pv.recs, g);
+    const SegRec rec = load_rec(pv.recs + (int64_t)(kListRows + 1) * plan_cap(nseg), blockIdx.x);
+    if ((int)blockIdx.x >= count) return;
     const int rows = rec.M, cols = rec.N;
     if (cols <= kRunCols) return;                       // the lane-run kernel's
     const int wave = uniform((int)(threadIdx.x >> 6));
@@ -374,15 +376,20 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
     // lane-run kernel: z spreads the 16-row strips over workgroups when there are few (segment, head) pairs
     int64_t z_runs = 4, z_rows = 8;
     bool rows_work = true;
+    int64_t n_rows = nseg;                               // length of the row kernel's list (grid)
     if (info) {
         nseg = info->nseg;
         const int64_t groups = (((int64_t)info->max_M + 15) / 16 + kSoftmaxWaves - 1) / kSoftmaxWaves;
         const int64_t want = ((int64_t)cus * 8 + nseg * args.H - 1) / std::max<int64_t>(1, nseg * args.H);
         z_runs = std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
-        rows_work = info->max_N > kRunCols;
-        // row kernel: about four workgroups' worth of rows in flight per compute unit, never more than one
-        // wavefront per row
-        z_rows = std::max<int64_t>(1, std::min<int64_t>(4 * want, (info->max_M + kSoftmaxWaves - 1) / kSoftmaxWaves));
+        n_rows = info->list_rows;
+        rows_work = n_rows > 0;
+        // row kernel: about four workgroups' worth of rows in flight per compute unit over ITS segments,
+        // never more than one wavefront per row
+        const int64_t pairs = std::max<int64_t>(1, n_rows * args.H);
+        const int64_t want_rows = ((int64_t)cus * 32 + pairs - 1) / pairs;
+        z_rows = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want_rows, 4096),
+                                                        (info->max_M + kSoftmaxWaves - 1) / kSoftmaxWaves));
     }
     if (nseg <= 0) return BA_OK;
     const dim3 grid_runs((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs);
@@ -392,7 +399,7 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
         hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 16>), grid_runs, dim3(kSoftmaxThreads), 0, stream, args);
     if (rows_work)
         hipLaunchKernelGGL((softmax_rows_kernel<DT, BACKWARD>),
-                           dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z_rows), dim3(kSoftmaxThreads), 0, stream,
+                           dim3((unsigned)n_rows, (unsigned)args.H, (unsigned)z_rows), dim3(kSoftmaxThreads), 0, stream,
                            args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }

@@ -73,7 +73,7 @@ typedef struct ba_plan_info {
     int32_t list_rest;      /* segment kernel: packs, element-wise class, leftovers */
     int32_t small_max_N;    /* widest segment of the strip kernel's main launch */
     int32_t small_max_M;    /* tallest segment of the strip kernel's main launch */
-    int32_t reserved;
+    int32_t list_rows;      /* softmax row kernel: segments with N > 256 (GEMM and softmax plans) */
 } ba_plan_info;
 
 const char *ba_status_string(int status);

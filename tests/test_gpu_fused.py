@@ -88,7 +88,7 @@ def test_long_k_and_every_launch_class(dev):
 
 
 def test_work_lists_match_the_shape_rules(dev):
-    # The lengths of the four work lists against the classification restated on the host.
+    # The lengths of the work lists against the classification restated on the host.
     for cfg in (1, 2, 3, 4, 5):
         w = workloads.make(cfg)
         plan = make_plan(dev, w.M, w.N, w.K)
@@ -103,3 +103,4 @@ def test_work_lists_match_the_shape_rules(dev):
         assert i.list_small <= small and small - i.list_small <= 2 * i.pack_items * 8, cfg   # packs take tiny ones
         assert i.list_tile == int(((w.N > 256) | ((w.N >= 128) & (blocks == 0))).sum()), cfg
         assert packed <= w.nseg
+        assert i.list_rows == int(((w.N > 256) & (w.M >= 1)).sum()), cfg     # the softmax row kernel's list
