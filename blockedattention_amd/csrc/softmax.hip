@@ -227,6 +227,36 @@ __global__ __launch_bounds__(kSoftmaxThreads, MAXG <= 8 ? 3 : 1) void softmax_ru
 
 // --------------------------------------------------------------------- rows
 // One wavefront per row; lane l owns columns 8*l .. 8*l+7 of every 512-column step.
+// Eight consecutive elements as they come from memory (any element alignment).
+template <int DT> struct Raw8 {
+    typedef typename Io<DT>::T T;
+    u32x4 a;
+    __device__ __forceinline__ void load(const T *p) { a = *reinterpret_cast<const u32x4_unaligned *>(p); }
+    __device__ __forceinline__ void unpack(float (&x)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { x[2 * i] = Io<DT>::lo(a[i]); x[2 * i + 1] = Io<DT>::hi(a[i]); }
+    }
+    static __device__ __forceinline__ void store(T *p, const float (&x)[8]) {
+        *reinterpret_cast<u32x4_unaligned *>(p) = u32x4{Io<DT>::pack(x[0], x[1]), Io<DT>::pack(x[2], x[3]),
+                                                        Io<DT>::pack(x[4], x[5]), Io<DT>::pack(x[6], x[7])};
+    }
+};
+template <> struct Raw8<BA_F32> {
+    typedef float T;
+    f32x4 a, b;
+    __device__ __forceinline__ void load(const T *p) {
+        a = *reinterpret_cast<const f32x4_unaligned *>(p);
+        b = *reinterpret_cast<const f32x4_unaligned *>(p + 4);
+    }
+    __device__ __forceinline__ void unpack(float (&x)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { x[i] = a[i]; x[4 + i] = b[i]; }
+    }
+    static __device__ __forceinline__ void store(T *p, const float (&x)[8]) {
+        *reinterpret_cast<f32x4_unaligned *>(p) = f32x4{x[0], x[1], x[2], x[3]};
+        *reinterpret_cast<f32x4_unaligned *>(p + 4) = f32x4{x[4], x[5], x[6], x[7]};
+    }
+};
 template <int DT>
 __device__ __forceinline__ void load_eight(const typename Io<DT>::T *p, int valid, float fill, float (&x)[8]) {
     typedef Io<DT> I;
@@ -264,6 +294,65 @@ __device__ __forceinline__ void store_eight(typename Io<DT>::T *p, int valid, co
     }
 }
 
+// Forward softmax of rows first, first + stride, ... of one segment whose rows take STEPS 512-column
+// steps (256 < cols <= 512 * STEPS); one wavefront per row, the whole row in registers.
+// Every step is one unconditional 8-element load per lane: a lane whose run would pass the end of the
+// row reads the eight elements ENDING at the row's end instead; the elements it shares with the lane
+// before get weight 0 in the sum and are stored again with the same value (lanes wholly past the end
+// repeat that last run).  Straight-line code: the loads of the next row are issued before the
+// arithmetic of the current one, and nothing waits for stores.
+template <int DT, int STEPS>
+__device__ __forceinline__ void softmax_rows_forward(const typename Io<DT>::T *src, typename Io<DT>::T *dst, int rows,
+                                                     int cols, int first, int stride, float c, float sgn) {
+    const int lane = lane_id();
+    int at[STEPS];                                       // first column of the lane's run in step k
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) at[k] = min(512 * k + 8 * lane, cols - 8);
+    // elements of the last step's run that belong to the lanes before (8 or more: none are ours)
+    const int own = 512 * (STEPS - 1) + 8 * lane - at[STEPS - 1];
+    float w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = (i >= own && own < 8) ? 1.f : 0.f;
+    Raw8<DT> raw[STEPS];
+    if (first < rows) {
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) raw[k].load(src + (int64_t)first * cols + at[k]);
+    }
+    for (int r = first; r < rows; r += stride) {
+        float v[STEPS][8];
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) raw[k].unpack(v[k]);
+        if (r + stride < rows) {
+#pragma unroll
+            for (int k = 0; k < STEPS; ++k) raw[k].load(src + (int64_t)(r + stride) * cols + at[k]);
+        }
+        float mx = -3.0e38f;
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k)
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) mx = max3(mx, sgn * v[k][i], sgn * v[k][i + 1]);
+        mx = wave_max(mx);
+        const float bias = -((__builtin_fabsf(mx) == INFINITY) ? 0.f : mx) * c;
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[k][i] = __builtin_amdgcn_exp2f(fmaf(sgn * v[k][i], c, bias));
+                sum = k < STEPS - 1 ? sum + v[k][i] : fmaf(v[k][i], w[i], sum);
+            }
+        sum = wave_sum(sum);
+        const float inv = __builtin_amdgcn_rcpf(sum);
+        typename Io<DT>::T *y = dst + (int64_t)r * cols;
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[k][i] *= inv;
+            Raw8<DT>::store(y + at[k], v[k]);
+        }
+    }
+}
+
 template <int DT, bool BACKWARD>
 __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxArgs a) {
     typedef typename Io<DT>::T T;
@@ -273,14 +362,21 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
     if (nseg < 0) return;
     const int count = (int)((ConstHdr)(uintptr_t)a.plan)->totals[kListRows];
     const PlanRO pv = plan_ro(a.plan, nseg);
-    const SegRec rec = load_rec(pv.recs + (int64_t)(kListRows + 1) * plan_cap(nseg), blockIdx.x);
-    if ((int)blockIdx.x >= count) return;
+    // Workgroups start in the order of their linear index.  Taking the row group from its fastest digits,
+    // then the head, then the list entry makes the machine work through one (segment, head) after the
+    // other, each as one stream of consecutive rows; with the entry fastest it would read and write
+    // hundreds of segments of unequal row lengths at once, which costs a third of the bandwidth.
+    const uint64_t lin = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
+    const unsigned group = (unsigned)(lin % gridDim.z), head = (unsigned)((lin / gridDim.z) % gridDim.y);
+    const unsigned entry = (unsigned)(lin / ((uint64_t)gridDim.z * gridDim.y));
+    const SegRec rec = load_rec(pv.recs + (int64_t)(kListRows + 1) * plan_cap(nseg), entry);
+    if ((int)entry >= count) return;
     const int rows = rec.M, cols = rec.N;
     if (cols <= kRunCols) return;                       // the lane-run kernel's
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int lane = lane_id();
-    const int first = blockIdx.z * kSoftmaxWaves + wave, stride = gridDim.z * kSoftmaxWaves;
-    const int64_t seg0 = (int64_t)blockIdx.y * a.Dsrc + rec.offO;
+    const int first = group * kSoftmaxWaves + wave, stride = gridDim.z * kSoftmaxWaves;
+    const int64_t seg0 = (int64_t)head * a.Dsrc + rec.offO;
     const T *src = reinterpret_cast<const T *>(a.src) + seg0;
     const T *aux = reinterpret_cast<const T *>(a.aux) + seg0;
     T *dst = reinterpret_cast<T *>(a.dst) + seg0;
@@ -289,49 +385,21 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
     const float c = c_signed * sgn;
     const int steps = (cols + 511) >> 9;
 
+    if (!BACKWARD && steps <= kRowSteps) {
+#define BA_ROWS(S_) case S_: softmax_rows_forward<DT, S_>(src, dst, rows, cols, first, stride, c, sgn); break;
+        switch (steps) {
+            BA_ROWS(1) BA_ROWS(2) BA_ROWS(3) BA_ROWS(4) BA_ROWS(5) BA_ROWS(6) BA_ROWS(7) BA_ROWS(8)
+            default: break;
+        }
+#undef BA_ROWS
+        return;
+    }
     for (int r = first; r < rows; r += stride) {
         const int64_t e0 = (int64_t)r * cols;
         const T *x = src + e0;
         T *y = dst + e0;
         if (!BACKWARD) {
-            if (steps <= kRowSteps) {
-                float v[kRowSteps][8];
-                float mx = -3.0e38f;
-#pragma unroll
-                for (int k = 0; k < kRowSteps; ++k) {
-                    if (k < steps) {
-                        const int col = 512 * k + 8 * lane;
-                        load_eight<DT>(x + col, cols - col, -3.0e38f * sgn, v[k]);
-#pragma unroll
-                        for (int i = 0; i < 8; i += 2) mx = max3(mx, sgn * v[k][i], sgn * v[k][i + 1]);
-                    }
-                }
-                mx = wave_max(mx);
-                const float bias = -((__builtin_fabsf(mx) == INFINITY) ? 0.f : mx) * c;
-                float sum = 0.f;
-#pragma unroll
-                for (int k = 0; k < kRowSteps; ++k) {
-                    if (k < steps) {
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) {
-                            v[k][i] = __builtin_amdgcn_exp2f(fmaf(sgn * v[k][i], c, bias));
-                            sum += v[k][i];
-                        }
-                    }
-                }
-                sum = wave_sum(sum);
-                if (c == 0.f) sum = (float)cols;           // scale 0: the padding slots counted as exp2(0) too
-                const float inv = __builtin_amdgcn_rcpf(sum);
-#pragma unroll
-                for (int k = 0; k < kRowSteps; ++k) {
-                    if (k < steps) {
-                        const int col = 512 * k + 8 * lane;
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) v[k][i] *= inv;
-                        store_eight<DT>(y + col, cols - col, v[k]);
-                    }
-                }
-            } else {
+            {
                 float mx = -INFINITY;
                 for (int col = lane; col < cols; col += 64) mx = fmaxf(mx, sgn * Io<DT>::ld(x + col));
                 mx = wave_max(mx);
