@@ -257,43 +257,6 @@ template <> struct Raw8<BA_F32> {
         *reinterpret_cast<f32x4_unaligned *>(p + 4) = f32x4{x[4], x[5], x[6], x[7]};
     }
 };
-template <int DT>
-__device__ __forceinline__ void load_eight(const typename Io<DT>::T *p, int valid, float fill, float (&x)[8]) {
-    typedef Io<DT> I;
-    if (valid >= 8) {
-        if constexpr (DT == BA_F32) {
-            const f32x4 lo = *reinterpret_cast<const f32x4_unaligned *>(p);
-            const f32x4 hi = *reinterpret_cast<const f32x4_unaligned *>(reinterpret_cast<const float *>(p) + 4);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { x[i] = lo[i]; x[4 + i] = hi[i]; }
-        } else {
-            const u32x4 v = *reinterpret_cast<const u32x4_unaligned *>(p);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { x[2 * i] = I::lo(v[i]); x[2 * i + 1] = I::hi(v[i]); }
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = i < valid ? I::ld(p + i) : fill;
-    }
-}
-template <int DT>
-__device__ __forceinline__ void store_eight(typename Io<DT>::T *p, int valid, const float (&x)[8]) {
-    typedef Io<DT> I;
-    if (valid >= 8) {
-        if constexpr (DT == BA_F32) {
-            *reinterpret_cast<f32x4_unaligned *>(p) = f32x4{x[0], x[1], x[2], x[3]};
-            *reinterpret_cast<f32x4_unaligned *>(reinterpret_cast<float *>(p) + 4) = f32x4{x[4], x[5], x[6], x[7]};
-        } else {
-            *reinterpret_cast<u32x4_unaligned *>(p) =
-                u32x4{I::pack(x[0], x[1]), I::pack(x[2], x[3]), I::pack(x[4], x[5]), I::pack(x[6], x[7])};
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (i < valid) I::st(p + i, x[i]);
-    }
-}
-
 // Forward softmax of rows first, first + stride, ... of one segment whose rows take STEPS 512-column
 // steps (256 < cols <= 512 * STEPS); one wavefront per row, the whole row in registers.
 // Every step is one unconditional 8-element load per lane: a lane whose run would pass the end of the
@@ -394,45 +357,93 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
 #undef BA_ROWS
         return;
     }
+    // Rows wider than the register path holds, and the backward: the row is streamed in 512-column steps,
+    // four steps of loads in flight, once per pass.  A lane reads the run of eight elements that starts
+    // at its column, or the run ENDING at the row's end when that would pass it; `own` is the number of
+    // leading elements of the run that belong to the lanes before (8 or more: none are this lane's).
+    // A lane writes only its own elements, so dst may alias src (or dy).
+    auto run_at = [&](int k, int &own) {
+        const int col = 512 * k + 8 * lane;
+        const int at = min(col, cols - 8);
+        own = col - at;
+        return at;
+    };
+    auto store_own = [&](T *p, const float (&v)[8], int own) {
+        if (own == 0) {
+            Raw8<DT>::store(p, v);
+        } else {
+#pragma unroll
+            for (int i = 1; i < 8; ++i)
+                if (i >= own) Io<DT>::st(p + i, v[i]);
+        }
+    };
+    // fn(k, at, own, x[8]) or, with a second source, fn(k, at, own, x[8], g[8]) for every step of the row
+    auto sweep = [&](const T *x, const T *g, auto &&fn) {
+        for (int k0 = 0; k0 < steps; k0 += 4) {
+            Raw8<DT> rx[4], rg[4];
+            int at[4], own[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (k0 + u < steps) {
+                    at[u] = run_at(k0 + u, own[u]);
+                    rx[u].load(x + at[u]);
+                    if (BACKWARD) rg[u].load(g + at[u]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (k0 + u < steps) {
+                    float xv[8], gv[8];
+                    rx[u].unpack(xv);
+                    if (BACKWARD) rg[u].unpack(gv);
+                    fn(at[u], own[u], xv, gv);
+                }
+            }
+        }
+    };
     for (int r = first; r < rows; r += stride) {
         const int64_t e0 = (int64_t)r * cols;
         const T *x = src + e0;
         T *y = dst + e0;
         if (!BACKWARD) {
-            {
-                float mx = -INFINITY;
-                for (int col = lane; col < cols; col += 64) mx = fmaxf(mx, sgn * Io<DT>::ld(x + col));
-                mx = wave_max(mx);
-                const float bias = -((mx == -INFINITY) ? 0.f : mx) * c;
-                float sum = 0.f;
-                for (int col = lane; col < cols; col += 64)
-                    sum += __builtin_amdgcn_exp2f(fmaf(sgn * Io<DT>::ld(x + col), c, bias));
-                sum = wave_sum(sum);
-                const float inv = 1.f / sum;
-                // src may alias dst: every lane re-reads only the elements it writes.
-                for (int col = lane; col < cols; col += 64)
-                    Io<DT>::st(y + col, __builtin_amdgcn_exp2f(fmaf(sgn * Io<DT>::ld(x + col), c, bias)) * inv);
-            }
+            float mx = -3.0e38f;
+            sweep(x, x, [&](int, int, const float (&xv)[8], const float (&)[8]) {
+#pragma unroll
+                for (int i = 0; i < 8; i += 2) mx = max3(mx, sgn * xv[i], sgn * xv[i + 1]);
+            });
+            mx = wave_max(mx);
+            const float bias = -((__builtin_fabsf(mx) == INFINITY) ? 0.f : mx) * c;
+            float sum = 0.f;
+            sweep(x, x, [&](int, int own, const float (&xv)[8], const float (&)[8]) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float p = __builtin_amdgcn_exp2f(fmaf(sgn * xv[i], c, bias));
+                    sum += i >= own ? p : 0.f;
+                }
+            });
+            sum = wave_sum(sum);
+            const float inv = __builtin_amdgcn_rcpf(sum);
+            sweep(x, x, [&](int at, int own, const float (&xv)[8], const float (&)[8]) {
+                float pv[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pv[i] = __builtin_amdgcn_exp2f(fmaf(sgn * xv[i], c, bias)) * inv;
+                store_own(y + at, pv, own);
+            });
         } else {
             // dx = scale * (dy - sum(y * dy)) * y; x is the saved forward output here.
             const T *dy = aux + e0;
             float dot = 0.f;
-            for (int col = 8 * lane; col < cols; col += 512) {
-                float yv[8], gv[8];
-                load_eight<DT>(x + col, cols - col, 0.f, yv);
-                load_eight<DT>(dy + col, cols - col, 0.f, gv);
+            sweep(x, dy, [&](int, int own, const float (&yv)[8], const float (&gv)[8]) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) dot = fmaf(yv[i], gv[i], dot);
-            }
+                for (int i = 0; i < 8; ++i) dot += i >= own ? yv[i] * gv[i] : 0.f;
+            });
             dot = wave_sum(dot);
-            for (int col = 8 * lane; col < cols; col += 512) {
-                float yv[8], gv[8];
-                load_eight<DT>(x + col, cols - col, 0.f, yv);
-                load_eight<DT>(dy + col, cols - col, 0.f, gv);
+            sweep(x, dy, [&](int at, int own, const float (&yv)[8], const float (&gv)[8]) {
+                float dv[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) yv[i] = a.scale * (gv[i] - dot) * yv[i];
-                store_eight<DT>(y + col, cols - col, yv);
-            }
+                for (int i = 0; i < 8; ++i) dv[i] = a.scale * (gv[i] - dot) * yv[i];
+                store_own(y + at, dv, own);
+            });
         }
     }
 }

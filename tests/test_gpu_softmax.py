@@ -63,6 +63,17 @@ def test_in_place_and_gapped_prefix_sum(dev):
     assert np.abs(out.float().cpu().numpy()[:, 16:] - ref[:, 16:]).max() < 1e-3
 
 
+def test_in_place_rows_wider_than_the_register_path(dev):
+    # 4613 = 9 * 512 + 5: the last step's run reaches back into columns the step before has already written.
+    rows, cols = [3, 2, 5], [4613, 513, 8200]
+    for dtype in (torch.float16, torch.float32):
+        src, out, plan = run_softmax(dev, rows, cols, 2, dtype, scale=0.3, seed=5)
+        buf = src.to(dev).clone()
+        capi.blocked_softmax(plan, buf, buf, 2, src.shape[1], 0.3)
+        assert torch.equal(buf, out)
+        assert_probs_close(out, oracle.per_segment_torch_softmax(src, rows, cols, 0.3), "wide in place")
+
+
 def test_all_neg_inf_row_is_nan_like_torch(dev):
     x = torch.tensor([[float("-inf")] * 4 + [0.0, float("-inf"), 1.0, 2.0]], dtype=torch.float32)
     plan = capi.plan_softmax(1, dev, dev_i64([2], dev), dev_i64([4], dev))
@@ -85,3 +96,20 @@ def test_backward_matches_oracle(dev, dtype):
     ref = oracle.blocked_softmax_backward(y.float().cpu().numpy(), dy.float().numpy(), rows, cols, 0.5)
     tol = 2e-3 if dtype == torch.float16 else 1e-6
     assert np.abs(dx.float().cpu().numpy() - ref).max() <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_backward_wide_ragged_rows_and_in_place(dev, dtype):
+    # row lengths around the 512-column steps (remainders 1, 5, 511, 0) and past the 4096-column register path
+    rows, cols = [2, 3, 1, 2, 2], [513, 4613, 1023, 1024, 300]
+    src, y, plan = run_softmax(dev, rows, cols, 2, dtype, scale=1.0, seed=11)
+    g = torch.Generator().manual_seed(12)
+    dy = torch.randn(y.shape, generator=g).to(dtype)
+    dx = torch.empty_like(y)
+    capi.blocked_softmax_backward(plan, y, dy.to(dev), dx, 2, y.shape[1], 1.0)
+    ref = oracle.blocked_softmax_backward(y.float().cpu().numpy(), dy.float().numpy(), rows, cols, 1.0)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-6
+    assert np.abs(dx.float().cpu().numpy() - ref).max() <= tol
+    buf = dy.to(dev).clone()                                   # dx written over dy
+    capi.blocked_softmax_backward(plan, y, buf, buf, 2, y.shape[1], 1.0)
+    assert torch.equal(buf, dx)
