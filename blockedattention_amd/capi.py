@@ -134,8 +134,11 @@ class Plan:
 
 
 def plan_gemm(nseg, device, MList=None, NList=None, KList=None, accum1=None, accum2=None, accumOut=None,
-              mode=None):
-    """Run the scheduler.  Tensors passed as None in an *output* role are not written."""
+              mode=None, plan=None):
+    """Run the scheduler.  Tensors passed as None in an *output* role are not written.
+
+    ``plan``: an existing Plan of the same segment count to schedule into again (no allocation, e.g.
+    under stream capture); its host summary is dropped, since it describes the previous schedule."""
     have_lists = MList is not None and NList is not None and KList is not None
     have_accum = accum1 is not None and accum2 is not None and accumOut is not None
     if mode is None:
@@ -144,7 +147,11 @@ def plan_gemm(nseg, device, MList=None, NList=None, KList=None, accum1=None, acc
                        (accum1, nseg + 1, "mat1Accum"), (accum2, nseg + 1, "mat2Accum"),
                        (accumOut, nseg + 1, "outAccum")):
         _meta(t, n, name)
-    plan = Plan(nseg, device)
+    if plan is None:
+        plan = Plan(nseg, device)
+    elif plan.nseg != int(nseg):
+        raise BlockedAttentionError(f"the plan was sized for {plan.nseg} segments, not {nseg}")
+    plan.info = None
     st = load().ba_plan_gemm(plan.ptr, plan.bytes, nseg, mode, _ptr(MList), _ptr(NList), _ptr(KList),
                              _ptr(accum1), _ptr(accum2), _ptr(accumOut), _stream())
     check(st, "ba_plan_gemm")

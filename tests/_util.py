@@ -65,14 +65,19 @@ def assert_probs_close(got, ref, what=""):
         assert diff.max().item() <= 1e-3, f"{what}: probabilities off by {float(diff.max())}"
 
 
-def run_all(dev, M, N, K, H, dtype, scale, seed=0, dist="normal", sigma=1.0, check_gemm=True, check_softmax=True):
-    """GEMM, fused pair and standalone softmax through the C ABI against the oracle."""
+def run_all(dev, M, N, K, H, dtype, scale, seed=0, dist="normal", sigma=1.0, check_gemm=True, check_softmax=True,
+            summary=True):
+    """GEMM, fused pair and standalone softmax through the C ABI against the oracle.
+
+    summary=False: the launches get no host copy of the plan summary (nothing was read back between the
+    scheduler and the kernels): grids are sized by the segment count alone and the kernels take the list
+    lengths from the plan on the device."""
     M = np.asarray(M, np.int64); N = np.asarray(N, np.int64); K = np.asarray(K, np.int64)
     A, B = random_operands(M, N, K, H, dtype, seed, dist, sigma)
-    plan = make_plan(dev, M, N, K)
-    info = plan.info
+    plan = make_plan(dev, M, N, K, read=summary)
     d1, d2, do = int((M * K).sum()), int((N * K).sum()), int((M * N).sum())
-    assert (info.Dm1, info.Dm2, info.Dout) == (d1, d2, do)
+    if summary:
+        assert (plan.info.Dm1, plan.info.Dm2, plan.info.Dout) == (d1, d2, do)
     sc, pr = oracle.per_segment_torch(A, B, M, N, K, scale, want="both")
     Ad, Bd = A.to(dev), B.to(dev)
     out = torch.full((H, do), float("nan"), dtype=dtype, device=dev)
@@ -86,5 +91,7 @@ def run_all(dev, M, N, K, H, dtype, scale, seed=0, dist="normal", sigma=1.0, che
         sm = torch.full((H, do), float("nan"), dtype=dtype, device=dev)
         capi.blocked_softmax(plan, out, sm, H, do, scale)
         assert_probs_close(sm, oracle.per_segment_torch_softmax(out.cpu(), M, N, scale), "softmax")
-    assert plan.read().run_errors == 0
+    assert plan.info is not None or not summary
+    info = plan.read()
+    assert info.run_errors == 0 and (info.Dm1, info.Dm2, info.Dout) == (d1, d2, do)
     return plan

@@ -104,3 +104,14 @@ def test_work_lists_match_the_shape_rules(dev):
         assert i.list_tile == int(((w.N > 256) | ((w.N >= 128) & (blocks == 0))).sum()), cfg
         assert packed <= w.nseg
         assert i.list_rows == int(((w.N > 256) & (w.M >= 1)).sum()), cfg     # the softmax row kernel's list
+
+
+def test_launches_without_the_host_summary(dev):
+    # Nothing is read back between the scheduler and the kernels: every kernel is launched over nseg slots
+    # with default z and finds its list (or nothing) in the plan.  All five lists, tall and wide segments.
+    M = [40, 130, 20, 64, 7, 5, 300, 33, 700, 12, 1]; N = [48, 300, 200, 256, 6, 9, 129, 64, 40, 5000, 1]
+    K = [160, 256, 200, 128, 16, 16, 136, 264, 64, 8, 8]
+    for dtype, scale in ((torch.float16, 0.05), (torch.bfloat16, -0.05)):
+        plan = run_all(dev, M, N, K, 2, dtype, scale, seed=5, summary=False)
+        i = plan.info
+        assert i.list_big == 1 and i.list_tile == 4 and i.list_rows == 2 and i.pack_items == 1
