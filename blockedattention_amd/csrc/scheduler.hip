@@ -148,13 +148,15 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         if (a.kind == 0 && __syncthreads_or(packable)) {
             sM[tid] = mi; sN[tid] = ni; sK[tid] = aligned ? ki : -1; sPack[tid] = 0;
             __syncthreads();
-            if ((tid & 15) == 0) {
+            // the window walkers sit side by side in the first wavefront(s): thread w walks window w
+            if (tid < kSchedThreads / 16) {
+                const int wbase = tid * 16;
                 int32_t wm[16], wn[16], wk[16];
 #pragma unroll
                 for (int j = 0; j < 16; j += 4) {
-                    const int4 vm = *reinterpret_cast<const int4 *>(&sM[tid + j]);
-                    const int4 vn = *reinterpret_cast<const int4 *>(&sN[tid + j]);
-                    const int4 vk = *reinterpret_cast<const int4 *>(&sK[tid + j]);
+                    const int4 vm = *reinterpret_cast<const int4 *>(&sM[wbase + j]);
+                    const int4 vn = *reinterpret_cast<const int4 *>(&sN[wbase + j]);
+                    const int4 vk = *reinterpret_cast<const int4 *>(&sK[wbase + j]);
                     wm[j] = vm.x; wm[j + 1] = vm.y; wm[j + 2] = vm.z; wm[j + 3] = vm.w;
                     wn[j] = vn.x; wn[j + 1] = vn.y; wn[j + 2] = vn.z; wn[j + 3] = vn.w;
                     wk[j] = vk.x; wk[j + 1] = vk.y; wk[j + 2] = vk.z; wk[j + 3] = vk.w;
@@ -184,10 +186,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
                     }
                 }
                 close();
-                sPack[tid] = (int32_t)follow;
-                sPack[tid + 1] = (int32_t)(uint32_t)lens_lo;
-                sPack[tid + 2] = (int32_t)(uint32_t)(lens_lo >> 32);
-                sPack[tid + 3] = (int32_t)(uint32_t)lens_hi;
+                sPack[wbase] = (int32_t)follow;
+                sPack[wbase + 1] = (int32_t)(uint32_t)lens_lo;
+                sPack[wbase + 2] = (int32_t)(uint32_t)(lens_lo >> 32);
+                sPack[wbase + 3] = (int32_t)(uint32_t)lens_hi;
             }
             __syncthreads();
             {
@@ -320,6 +322,7 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
     SchedArgs args{plan, nseg, mode, kind, M, N, K, a1, a2, aO};
     if (nseg <= 64) hipLaunchKernelGGL(schedule_kernel<64>, dim3(1), dim3(64), 0, stream, args);
     else if (nseg <= 256) hipLaunchKernelGGL(schedule_kernel<256>, dim3(1), dim3(256), 0, stream, args);
+    else if (nseg <= 512) hipLaunchKernelGGL(schedule_kernel<512>, dim3(1), dim3(512), 0, stream, args);
     else hipLaunchKernelGGL(schedule_kernel<kSchedThreadsMax>, dim3(1), dim3(kSchedThreadsMax), 0, stream, args);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
