@@ -87,8 +87,6 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     constexpr int kSchedWaves = kSchedThreads / 64;
     __shared__ int64_t sScan64[kSchedWaves * 3];
     __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
-    __shared__ __attribute__((aligned(16))) int32_t sM[kSchedThreads], sN[kSchedThreads], sK[kSchedThreads];
-    __shared__ int32_t sPack[kSchedThreads];
     __shared__ int32_t sRed[kSchedWaves][6];
 
     const int tid = threadIdx.x;
@@ -146,60 +144,33 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         // Only batches that contain segments small enough to pack pay for the window walk.
         const bool packable = aligned && mi >= 1 && ni >= 1 && ki >= 1 && mi < kPackDim && ni < kPackDim;
         if (a.kind == 0 && __syncthreads_or(packable)) {
-            sM[tid] = mi; sN[tid] = ni; sK[tid] = aligned ? ki : -1; sPack[tid] = 0;
-            __syncthreads();
-            // the window walkers sit side by side in the first wavefront(s): thread w walks window w
-            if (tid < kSchedThreads / 16) {
-                const int wbase = tid * 16;
-                int32_t wm[16], wn[16], wk[16];
+            // A window is the 16 lanes of one DPP row.  The greedy walk runs along the row: lane j takes the
+            // state that lane j-1 holds (rows sum, columns sum, members so far, K of the open pack), decides
+            // whether its segment joins that pack, and holds the state after it.  After step t lanes 0..t
+            // are final; every lane recomputes in every step, so nothing diverges and nothing leaves the
+            // registers.  Sizes enter clamped to 17 ("does not fit whatever follows").
+            const bool ok = mi >= 1 && ni >= 1 && ki >= 1 && aligned;
+            const uint32_t mc = (uint32_t)min(mi, kPackDim + 1), nc = (uint32_t)min(ni, kPackDim + 1);
+            const uint32_t alone = mc | (nc << 8) | ((ok ? 1u : 0u) << 16);   // a pack opened by this segment
+            uint32_t st = alone;
+            int32_t kopen = ki;
+            bool joins = false;
 #pragma unroll
-                for (int j = 0; j < 16; j += 4) {
-                    const int4 vm = *reinterpret_cast<const int4 *>(&sM[wbase + j]);
-                    const int4 vn = *reinterpret_cast<const int4 *>(&sN[wbase + j]);
-                    const int4 vk = *reinterpret_cast<const int4 *>(&sK[wbase + j]);
-                    wm[j] = vm.x; wm[j + 1] = vm.y; wm[j + 2] = vm.z; wm[j + 3] = vm.w;
-                    wn[j] = vn.x; wn[j + 1] = vn.y; wn[j + 2] = vn.z; wn[j + 3] = vn.w;
-                    wk[j] = vk.x; wk[j + 1] = vk.y; wk[j + 2] = vk.z; wk[j + 3] = vk.w;
-                }
-                // follow: bit j = entry j joins the pack before it; lens: 5 bits per entry = pack length at
-                // its leader.  Both stay in registers; the window's lanes decode them after the barrier.
-                uint32_t follow = 0;
-                uint64_t lens_lo = 0, lens_hi = 0;              // entries 0..11 / 12..15
-                int start = 0, len = 0, sumM = 0, sumN = 0, kcur = 0;
-                auto close = [&]() {
-                    if (len >= 2) {
-                        if (start < 12) lens_lo |= (uint64_t)len << (5 * start);
-                        else lens_hi |= (uint64_t)len << (5 * (start - 12));
-                    }
-                };
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    const bool ok = wm[j] >= 1 && wn[j] >= 1 && wk[j] >= 1;
-                    const bool fits = ok && len > 0 && wk[j] == kcur && sumM + wm[j] <= kPackDim &&
-                                      sumN + wn[j] <= kPackDim;
-                    if (fits) {
-                        sumM += wm[j]; sumN += wn[j]; ++len;
-                        follow |= 1u << j;
-                    } else {
-                        close();
-                        start = j; len = ok ? 1 : 0; sumM = wm[j]; sumN = wn[j]; kcur = wk[j];
-                    }
-                }
-                close();
-                sPack[wbase] = (int32_t)follow;
-                sPack[wbase + 1] = (int32_t)(uint32_t)lens_lo;
-                sPack[wbase + 2] = (int32_t)(uint32_t)(lens_lo >> 32);
-                sPack[wbase + 3] = (int32_t)(uint32_t)lens_hi;
+            for (int t = 1; t < 16; ++t) {
+                const uint32_t pst = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)st, 0x111, 0xf, 0xf, false);
+                const int32_t pk = __builtin_amdgcn_update_dpp(0, kopen, 0x111, 0xf, 0xf, false);
+                const uint32_t sm = (pst & 0xff) + mc, sn = ((pst >> 8) & 0xff) + nc, len = pst >> 16;
+                joins = ok && len > 0 && pk == ki && sm <= (uint32_t)kPackDim && sn <= (uint32_t)kPackDim;
+                st = joins ? (sm | (sn << 8) | ((len + 1) << 16)) : alone;
+                kopen = ki;                                   // a joining segment has the pack's K anyway
             }
-            __syncthreads();
-            {
-                const int wbase = tid & ~15, j = tid & 15;
-                const uint32_t follow = (uint32_t)sPack[wbase];
-                const uint64_t lens_lo = (uint32_t)sPack[wbase + 1] | ((uint64_t)(uint32_t)sPack[wbase + 2] << 32);
-                const uint64_t lens_hi = (uint32_t)sPack[wbase + 3];
-                const int len = (int)((j < 12 ? lens_lo >> (5 * j) : lens_hi >> (5 * (j - 12))) & 31);
-                pack = ((follow >> j) & 1) ? -1 : len;
-            }
+            // members of a pack = this leader plus the run of joining lanes right after it
+            const uint64_t jb = __ballot(joins);
+            const int j = lane & 15;
+            const uint32_t row = (uint32_t)(jb >> (lane & 48)) & 0xffffu;
+            const uint32_t after = (~row & 0xffffu) >> (j + 1);              // bit i: lane j+1+i does not join
+            const int run = j == 15 ? 0 : min((int)__builtin_ctz(after | (1u << (15 - j))), 15 - j);
+            pack = joins ? -1 : (ok && run >= 1) ? run + 1 : 0;
         }
 
         const int32_t strips = (ni >= 1) ? (mi + kStripRows - 1) / kStripRows : 0;
