@@ -257,7 +257,12 @@ def main():
         import blockedAttention
         ML, NL, KL = case.M, case.N, case.K
         op = lambda: blockedAttention.blockGEMMSoftmax(case.A, case.B, MList=ML, NList=NL, KList=KL, scale=w.scale)
+        # the operator as a model calls it, layer after layer with the batch's metadata tensors: the schedule
+        # of the first call is reused; and with that cache off (scheduler + one host synchronisation per call)
         line["detail"]["torch_op_us"] = round(case.wall_us(op, max(10, args.steps // 4), 5), 3)
+        blockedAttention.set_schedule_cache(0)
+        line["detail"]["torch_op_uncached_us"] = round(case.wall_us(op, max(10, args.steps // 4), 5), 3)
+        blockedAttention.set_schedule_cache(8)
     except ImportError as e:
         line["detail"]["torch_op_us"] = f"extension not built: {e}"
     if not args.no_cpu:

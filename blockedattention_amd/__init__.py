@@ -6,7 +6,7 @@ Importing the operators needs the in-tree build (``python -m
 blockedattention_amd.build``); nothing falls back to PyTorch or the CPU.
 """
 
-__all__ = ["blockGEMM", "blockSoftmax", "blockGEMMSoftmax"]
+__all__ = ["blockGEMM", "blockSoftmax", "blockGEMMSoftmax", "set_schedule_cache", "schedule_cache_stats"]
 
 
 def __getattr__(name):

@@ -68,3 +68,17 @@ def blockGEMMSoftmax(
     """
     return blockAttention.sparseBlockedGEMMSoftmax(mat1, mat2, mat1Accum, mat2Accum, outAccum, MList, NList, KList,
                                                    float(scale), bool(out_fp32))
+
+
+def set_schedule_cache(capacity: int) -> None:
+    """How many schedules the operators keep for metadata tensors they have seen (default 8; 0 = off).
+
+    A call whose metadata tensors are the same objects, unmodified (PyTorch's version counters), as in an
+    earlier call reuses that call's device-side plan and skips the scheduler and its host synchronisation.
+    Turn it off only if metadata tensors are rewritten through raw pointers, which PyTorch cannot see."""
+    blockAttention.set_schedule_cache(int(capacity))
+
+
+def schedule_cache_stats() -> dict:
+    hits, misses, entries, capacity = blockAttention.schedule_cache_stats()
+    return {"hits": hits, "misses": misses, "entries": entries, "capacity": capacity}

@@ -12,9 +12,19 @@
 //
 // Every precondition the reference leaves to assert() is a TORCH_CHECK here.
 // The tensors are used as device memory only; all work happens in
-// libblockedattn_hip.so on the current HIP stream.  One host synchronisation
-// per call: reading the plan summary, which carries Dout (needed to allocate
-// the result) and the device-side metadata verdict.
+// libblockedattn_hip.so on the current HIP stream.  Scheduling costs one host
+// synchronisation: reading the plan summary, which carries Dout (needed to
+// allocate the result) and the device-side metadata verdict.  The layers and
+// heads of a model call these operators many times with the SAME metadata
+// tensors, so the last few schedules are kept, keyed by the identity and the
+// version counter of every metadata tensor: a repeated call launches its
+// kernels at once.  set_schedule_cache(0) turns that off (needed only by a
+// caller that rewrites metadata tensors behind PyTorch's back, through raw
+// pointers, which the version counters cannot see).
+#include <array>
+#include <deque>
+#include <mutex>
+
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
@@ -68,6 +78,86 @@ struct Schedule {
     ba_plan_info info;
 };
 
+// ---------------------------------------------------------------- schedule cache
+struct ScheduleKey {
+    int kind = 0;                                   // 0 GEMM, 1 softmax
+    int device = -1;
+    std::array<const void *, 6> impl{};             // TensorImpl of each metadata tensor (nullptr: not given)
+    std::array<int64_t, 6> version{};
+    bool cacheable = true;
+    bool operator==(const ScheduleKey &o) const {
+        return kind == o.kind && device == o.device && impl == o.impl && version == o.version;
+    }
+};
+
+ScheduleKey make_key(int kind, const Tensor &like, std::initializer_list<const OptTensor *> metas) {
+    ScheduleKey k;
+    k.kind = kind;
+    k.device = like.device().index();
+    size_t i = 0;
+    for (const OptTensor *m : metas) {
+        if (m->has_value() && (*m)->defined()) {
+            if ((*m)->is_inference()) k.cacheable = false;      // no version counter to watch
+            else { k.impl[i] = (*m)->unsafeGetTensorImpl(); k.version[i] = (int64_t)(*m)->_version(); }
+        }
+        ++i;
+    }
+    return k;
+}
+
+struct ScheduleCache {
+    std::mutex mu;
+    std::deque<std::pair<ScheduleKey, Schedule>> entries;       // most recent first; entries keep their tensors alive
+    size_t capacity = 8;
+    int64_t hits = 0, misses = 0;
+};
+ScheduleCache &cache() {
+    static ScheduleCache c;
+    return c;
+}
+
+bool cache_lookup(const ScheduleKey &key, Schedule &out) {
+    ScheduleCache &c = cache();
+    std::lock_guard<std::mutex> lock(c.mu);
+    if (c.capacity == 0 || !key.cacheable) return false;
+    for (auto it = c.entries.begin(); it != c.entries.end(); ++it) {
+        if (it->first == key) {
+            out = it->second;
+            if (it != c.entries.begin()) {
+                auto e = *it;
+                c.entries.erase(it);
+                c.entries.push_front(std::move(e));
+            }
+            ++c.hits;
+            return true;
+        }
+    }
+    ++c.misses;
+    return false;
+}
+
+void cache_store(const ScheduleKey &key, const Schedule &s) {
+    ScheduleCache &c = cache();
+    std::lock_guard<std::mutex> lock(c.mu);
+    if (c.capacity == 0 || !key.cacheable) return;
+    c.entries.emplace_front(key, s);
+    while (c.entries.size() > c.capacity) c.entries.pop_back();
+}
+
+void set_schedule_cache(int64_t capacity) {
+    TORCH_CHECK(capacity >= 0 && capacity <= 1024, "schedule cache capacity must be in [0, 1024]");
+    ScheduleCache &c = cache();
+    std::lock_guard<std::mutex> lock(c.mu);
+    c.capacity = (size_t)capacity;
+    while (c.entries.size() > c.capacity) c.entries.pop_back();
+}
+
+std::vector<int64_t> schedule_cache_stats() {
+    ScheduleCache &c = cache();
+    std::lock_guard<std::mutex> lock(c.mu);
+    return {c.hits, c.misses, (int64_t)c.entries.size(), (int64_t)c.capacity};
+}
+
 // The three metadata cases of the reference (cpp:17-44), resolved on the device.
 Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor &a2, const OptTensor &aO,
                        const OptTensor &M, const OptTensor &N, const OptTensor &K) {
@@ -76,6 +166,8 @@ Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor 
     TORCH_CHECK(have_accum || have_lists,
                 "sparseBlockedGEMM needs either (mat1Accum, mat2Accum, outAccum) or (MList, NList, KList)");
     Schedule s;
+    const ScheduleKey key = make_key(0, like, {&a1, &a2, &aO, &M, &N, &K});
+    if (cache_lookup(key, s)) return s;
     int64_t nseg;
     int mode;
     const auto opts = at::TensorOptions().dtype(at::kLong).device(like.device());
@@ -113,11 +205,15 @@ Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor 
     TORCH_CHECK(st != BA_ERR_BAD_METADATA, "segment metadata rejected: ", s.info.bad_segments,
                 " segment(s) have negative, oversized or inconsistent shapes / prefix sums");
     check_status(st, "ba_plan_read");
+    cache_store(key, s);
     return s;
 }
 
 Schedule schedule_softmax(const Tensor &like, const Tensor &rows, const Tensor &cols, const OptTensor &accum) {
     Schedule s;
+    const OptTensor rows_o(rows), cols_o(cols), none;
+    const ScheduleKey key = make_key(1, like, {&rows_o, &cols_o, &accum, &none, &none, &none});
+    if (cache_lookup(key, s)) return s;
     const int64_t nseg = rows.numel();
     check_meta(rows, "rowList", like, nseg); check_meta(cols, "colList", like, nseg);
     s.M = rows; s.N = cols;
@@ -137,6 +233,7 @@ Schedule schedule_softmax(const Tensor &like, const Tensor &rows, const Tensor &
     TORCH_CHECK(st != BA_ERR_BAD_METADATA, "segment metadata rejected: ", s.info.bad_segments,
                 " segment(s) have negative or oversized shapes or a prefix sum too small for them");
     check_status(st, "ba_plan_read");
+    cache_store(key, s);
     return s;
 }
 
@@ -278,4 +375,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sparseBlockedSoftmax", &sparseBlockedSoftmax_op, "sparseBlockedSoftmax forward");
     m.def("sparseBlockedSoftmaxScaled", &sparseBlockedSoftmaxScaled_op, "sparseBlockedSoftmax with a fused scale");
     m.def("sparseBlockedGEMMSoftmax", &sparseBlockedGEMMSoftmax_op, "fused sparseBlockedGEMM + softmax forward");
+    m.def("set_schedule_cache", &set_schedule_cache, "number of schedules kept for repeated metadata (0 = off)");
+    m.def("schedule_cache_stats", &schedule_cache_stats, "[hits, misses, entries, capacity]");
 }

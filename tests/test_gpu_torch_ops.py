@@ -113,3 +113,36 @@ def test_autograd_matches_per_segment_torch(dev):
     torch.testing.assert_close(probs.detach().cpu(), ref.detach(), rtol=1e-4, atol=1e-6)
     torch.testing.assert_close(A.grad.cpu(), Ar.grad, rtol=1e-3, atol=1e-5)
     torch.testing.assert_close(B.grad.cpu(), Br.grad, rtol=1e-3, atol=1e-5)
+
+
+def test_repeated_metadata_reuses_the_schedule(dev):
+    import blockedAttention
+    blockedAttention.set_schedule_cache(8)
+    M = [33, 7, 120, 64]; K = [64] * 4
+    A, B = random_operands(M, M, K, 2, torch.float16, seed=2)
+    Ad, Bd = A.to(dev), B.to(dev)
+    ML, KL = dl(M, dev), dl(K, dev)
+    ref = oracle.per_segment_torch(A, B, M, M, K, 0.125, want="probs")
+    before = blockedAttention.schedule_cache_stats()
+    for _ in range(3):                                   # e.g. one call per layer with the batch's metadata
+        assert_probs_close(blockedAttention.blockGEMMSoftmax(Ad, Bd, MList=ML, NList=ML, KList=KL, scale=0.125), ref, "cached")
+    after = blockedAttention.schedule_cache_stats()
+    assert after["misses"] - before["misses"] == 1 and after["hits"] - before["hits"] == 2
+    # an in-place change of a metadata tensor is seen through its version counter: new schedule, new result
+    M2 = [33, 7, 120, 32]
+    ML[3] = 32
+    A2, B2 = random_operands(M2, M2, K, 2, torch.float16, seed=3)
+    out = blockedAttention.blockGEMMSoftmax(A2.to(dev), B2.to(dev), MList=ML, NList=ML, KList=KL, scale=0.125)
+    assert_probs_close(out, oracle.per_segment_torch(A2, B2, M2, M2, K, 0.125, want="probs"), "after the change")
+    assert blockedAttention.schedule_cache_stats()["misses"] - after["misses"] == 1
+    # GEMM, softmax and the backward share the cache through their own keys
+    sc = blockedAttention.blockGEMM(A2.to(dev), B2.to(dev), None, None, None, ML, ML, KL)
+    pr = blockedAttention.blockSoftmax(sc, ML, ML)
+    pr2 = blockedAttention.blockSoftmax(sc, ML, ML)
+    assert torch.equal(pr, pr2)
+    blockedAttention.set_schedule_cache(0)
+    off = blockedAttention.schedule_cache_stats()
+    blockedAttention.blockSoftmax(sc, ML, ML)
+    now = blockedAttention.schedule_cache_stats()
+    assert (now["hits"], now["misses"], now["entries"]) == (off["hits"], off["misses"], 0)
+    blockedAttention.set_schedule_cache(8)
