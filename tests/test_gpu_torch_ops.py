@@ -146,3 +146,43 @@ def test_repeated_metadata_reuses_the_schedule(dev):
     now = blockedAttention.schedule_cache_stats()
     assert (now["hits"], now["misses"], now["entries"]) == (off["hits"], off["misses"], 0)
     blockedAttention.set_schedule_cache(8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_autograd_16bit_through_the_repacked_gemms(dev, dtype):
+    # dA = dS B (reduction over N) and dB = dS^T A (over M) with N, M that are not multiples of 8
+    import blockedAttention
+    M, N, K = [5, 33, 16, 130], [7, 20, 64, 257], [8, 16, 24, 64]
+    g = torch.Generator().manual_seed(4)
+    A0 = torch.randn((2, int(np.dot(M, K))), generator=g).to(dtype); B0 = torch.randn((2, int(np.dot(N, K))), generator=g).to(dtype)
+    ML, NL, KL = dl(M, dev), dl(N, dev), dl(K, dev)
+    A = A0.to(dev).requires_grad_(); B = B0.to(dev).requires_grad_()
+    out = blockedAttention.blockGEMM(A, B, MList=ML, NList=NL, KList=KL)
+    wgt = torch.randn(out.shape, generator=g).to(dtype)
+    for _ in range(2):                                           # the second pass reuses the derived schedules
+        A.grad = None; B.grad = None
+        out.backward(wgt.to(dev), retain_graph=True)
+    o1 = o2 = oo = 0
+    for m, n, k in zip(M, N, K):
+        a = A0[:, o1:o1 + m * k].reshape(2, m, k).float(); b = B0[:, o2:o2 + n * k].reshape(2, n, k).float()
+        ds = wgt[:, oo:oo + m * n].reshape(2, m, n).float()
+        assert_scores_close(A.grad[:, o1:o1 + m * k].reshape(2, m, k), ds @ b, f"dA {m}x{n}x{k}")
+        assert_scores_close(B.grad[:, o2:o2 + n * k].reshape(2, n, k), ds.transpose(1, 2) @ a, f"dB {m}x{n}x{k}")
+        o1 += m * k; o2 += n * k; oo += m * n
+    assert A.grad.dtype == dtype and A.grad.shape == A.shape and B.grad.shape == B.shape
+
+
+def test_transposed_and_unaligned_forward_16bit(dev):
+    import blockedAttention
+    M, N, K = [9, 100, 64, 3], [17, 40, 64, 300], [12, 70, 64, 20]           # K not multiples of 8
+    g = torch.Generator().manual_seed(6)
+    a = [torch.randn((2, m, k), generator=g).half() for m, k in zip(M, K)]
+    b = [torch.randn((2, n, k), generator=g).half() for n, k in zip(N, K)]
+    ref = torch.cat([(x.float() @ y.float().transpose(1, 2)).reshape(2, -1) for x, y in zip(a, b)], 1)
+    ML, NL, KL = dl(M, dev), dl(N, dev), dl(K, dev)
+    for t1 in (False, True):
+        for t2 in (False, True):
+            A = torch.cat([(x.transpose(1, 2) if t1 else x).reshape(2, -1) for x in a], 1).contiguous().to(dev)
+            B = torch.cat([(y.transpose(1, 2) if t2 else y).reshape(2, -1) for y in b], 1).contiguous().to(dev)
+            out = blockedAttention.blockGEMM(A, B, None, None, None, ML, NL, KL, t1, t2)
+            assert_scores_close(out, ref, f"transpose1={t1} transpose2={t2}")
