@@ -158,7 +158,10 @@ int launch_repack(const void *src_plan, int src_which, int swap_dims, int column
         const int64_t cols = dst_info->max_K;
         const int64_t units = column_major ? ((rows + 63) / 64) * ((cols + 63) / 64) : (rows * ((cols + 7) / 8) + 255) / 256;
         const int64_t want = ((int64_t)device_cu_count() * 8 + nseg * H - 1) / (nseg * H);
-        z = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(units, want), 1024));
+        // enough workgroups to fill the machine, and never more than eight tiles of the largest segment in
+        // one workgroup (workgroups past a segment's last tile leave at once)
+        z = std::max<int64_t>(std::min<int64_t>(units, want), std::min<int64_t>((units + 7) / 8, 64));
+        z = std::max<int64_t>(1, std::min<int64_t>(z, 1024));
     }
     RepackArgs a{src_plan, dst_plan, (const uint16_t *)src, (uint16_t *)dst, Dsrc, Ddst, (int)nseg,
                  src_which, dst_which, swap_dims, column_major};
