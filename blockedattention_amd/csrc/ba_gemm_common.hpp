@@ -30,6 +30,28 @@ __device__ __forceinline__ SegRes make_res(const Seg &s, const void *A, const vo
     return r;
 }
 
+// The compiler pads the distance between a matrix instruction and ITS OWN vector instructions that
+// read the result registers; instructions inside inline assembly (max3 below, the DPP reductions) get
+// no such padding, and one that reads an accumulator too soon after the last MFMA sees what the
+// register held before.  Call this between the MFMAs and the first inline-assembly read of acc: the
+// accumulators pass through 24 idle cycles (the longest write-back distance of these MFMAs is 18).
+template <int N>
+__device__ __forceinline__ void settle_mfma(f32x4 (&acc)[N]) {
+#pragma unroll
+    for (int g = 0; g < N; g += 8) {
+        if constexpr (N >= 8) {
+            const int b = g + 8 <= N ? g : N - 8;           // the last group may overlap the one before
+            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7"
+                         : "+v"(acc[b]), "+v"(acc[b + 1]), "+v"(acc[b + 2]), "+v"(acc[b + 3]), "+v"(acc[b + 4]),
+                           "+v"(acc[b + 5]), "+v"(acc[b + 6]), "+v"(acc[b + 7]));
+        } else {
+#pragma unroll
+            for (int k = 0; k + 1 < N; ++k) asm volatile("" : "+v"(acc[k]));
+            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+v"(acc[N - 1]));
+        }
+    }
+}
+
 __device__ __forceinline__ float max3(float a, float b, float c) {
     float r;   // one instruction for two new elements; fmaxf() would add a canonicalising max per operand
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
@@ -67,8 +89,10 @@ __device__ __forceinline__ void row16_sum4(float (&x)[4]) { BA_ROT_REDUCE("v_add
 // together hold whole rows.  In: scores, c >= 0 (scale * log2 e), w[g] in {0, 1} = whether the
 // column counts in the row sum (0 for columns a neighbouring lane also holds, or that do not exist;
 // such columns must hold a value that does not exceed the row maximum).  Out: probabilities.
-template <int G>
+// FROM_MFMA: acc comes straight out of matrix instructions (see settle_mfma).
+template <int G, bool FROM_MFMA = true>
 __device__ __forceinline__ void softmax_lane_runs(f32x4 (&acc)[G], const float (&w)[G], float c) {
+    if constexpr (FROM_MFMA) settle_mfma(acc);
     float ext[4], sum[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {

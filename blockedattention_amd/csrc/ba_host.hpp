@@ -27,6 +27,7 @@ struct RunArgs {
     int lds_blocks;   // 1 KiB operand blocks of dynamic LDS given to the segment / strip kernel
     int list;         // work list the launch walks (PrefixKind), or -1: every segment, by block index
     int nseg;         // segment count the plan was built for (checked against the plan)
+    int lds_extra;    // bytes of dynamic LDS behind the operand blocks (strip kernel: copy of the ragged run)
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,

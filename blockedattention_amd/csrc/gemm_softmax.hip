@@ -126,6 +126,7 @@ __device__ __forceinline__ void prepare_scores(f32x4 (&acc)[kMaxTiles], int nt, 
 // l = the row sum of acc.
 template <int NT>
 __device__ __forceinline__ void local_softmax(f32x4 (&acc)[kMaxTiles], int nt, float c, float &m, float &l) {
+    settle_mfma(acc);
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -292,6 +293,7 @@ __device__ __forceinline__ void wave_pack(const PlanRO &pv, int g, int len, int6
 // construction, no padding or swizzle to compute.  Segments whose B_g exceeds
 // the LDS window are walked in K slabs.
 constexpr int kLdsBlockBytes = 1024;
+constexpr int kRaggedCopyBytes = 16 * 256 + 1024;  // 16 rows of 128 k, and the round-up of the image to whole KiB
 constexpr int kSegWaves = 4;
 constexpr int kSegThreads = 64 * kSegWaves;
 // k-steps (of 32) whose A fragments a wavefront keeps in registers: 4 in the 128-register build, 2 in the
@@ -414,7 +416,16 @@ __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, c
 // value by 1 or 0 (w[g]) so overlapped and repeated columns count once; the row
 // maximum needs no mask at all.
 
-template <int DT, int G, bool FUSED, bool F32OUT>
+//
+// B_g in LDS, two layouts.  NAT = 0 (any K <= 128): blocks in MFMA operand order, filled by lanes that
+// each fetch the 16 bytes they will read (conflict-free linear reads; the fill gathers 64-byte pieces
+// of rows G apart).  NAT = 1 (K = 64) and NAT = 2 (K = 128): B_g as it lies in memory, so the fill is a
+// straight coalesced copy; inside every 256-byte window (two rows, or one) the sixteen 16-byte pieces
+// are XOR-permuted by the column slot j = row / G their rows belong to, and since the sixteen lanes
+// that read one operand together hold the same piece of rows G apart, i.e. of sixteen different slots
+// j, they fall into sixteen different bank groups.  The run [N-G, N) of the lane at the ragged end
+// (and of the lanes after it) is copied once more, unpermuted, behind the image and read from there.
+template <int DT, int G, bool FUSED, bool F32OUT, int NAT>
 __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, unsigned char *lds, int wave,
                                              int first_strip, int strip_step) {
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
@@ -441,9 +452,11 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
     };
     load_a(first_strip);
 
-    // ---- B_g -> LDS, block (ks, g) at (ks * G + g) KiB, in MFMA operand order:
-    //      lane (slot j, k-group rg) brings 16 bytes of B_g row col0 + g
-    {
+    // per (column tile g, k-step ks) the operand of this lane is read at vb[variant] + immediate
+    const unsigned char *vb[4];
+    if constexpr (NAT == 0) {
+        // ---- B_g -> LDS, block (ks, g) at (ks * G + g) KiB, in MFMA operand order:
+        //      lane (slot j, k-group rg) brings 16 bytes of B_g row col0 + g
         const uint16_t *bseg = (const uint16_t *)a.B + s.b;
         const int brow0 = owner ? col0 : N - 1;
         const int bstep = owner ? 1 : 0;
@@ -457,6 +470,39 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
                                              (__attribute__((address_space(3))) void *)(lds + b * kLdsBlockBytes),
                                              16, 0, 0);
         }
+        vb[0] = vb[1] = vb[2] = vb[3] = lds + lane * 16;
+    } else {
+        // ---- B_g -> LDS as it lies in memory: position p (16-byte pieces) of the image takes piece
+        //      (p & ~15) | ((p & 15) ^ key) of B_g, key = column slot of the window's rows
+        constexpr int kPieces = NAT == 1 ? 8 : 16;              // 16-byte pieces per row of B_g
+        const uint16_t *bseg = (const uint16_t *)a.B + s.b;
+        // Every instruction runs with all 64 lanes (1 KiB of LDS each): lanes past the end of B_g fetch its
+        // last piece into positions nobody reads, so the image takes whole KiB and the copy of the ragged
+        // run starts on the next KiB.
+        const int total = N * kPieces, padded = (total + 63) & ~63;
+        for (int p0 = wave * 64; p0 < padded; p0 += kSegWaves * 64) {
+            const int p = p0 + lane, w = p >> 4;
+            const int key = ((NAT == 1 ? 2 * w : w) / G) & 15;
+            const int piece = min((p & ~15) | ((p & 15) ^ key), total - 1);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bseg + piece * 8),
+                                             (__attribute__((address_space(3))) void *)(lds + p0 * 16), 16, 0, 0);
+        }
+        unsigned char *tail = lds + padded * 16;
+        const int tail_pieces = G * kPieces;
+        const int tail_key = J & 15;         // no lane with a full run uses this key: the copy's readers collide with none
+        for (int p0 = wave * 64; p0 < tail_pieces; p0 += kSegWaves * 64) {
+            const int q = p0 + lane;
+            const int p = min((q & ~15) | ((q & 15) ^ tail_key), tail_pieces - 1);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(bseg + ((N - G) * kPieces + p) * 8),
+                (__attribute__((address_space(3))) void *)(tail + p0 * 16), 16, 0, 0);
+        }
+        // rows of this lane: G*j + g in the image (full runs), or g of the copy of the last G rows
+        const bool full = j < J;
+        const unsigned char *base = full ? lds + (NAT == 1 ? 128 : 256) * (G * j) : tail;
+        const int kj = full ? j : tail_key;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) vb[c] = base + 64 * (c ^ (kj >> 2)) + 16 * (rg ^ (kj & 3));
     }
     // weights of the row sum: 1 for columns this lane alone accounts for
     float w[G];
@@ -467,7 +513,12 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
-    const unsigned char *blk = lds + lane * 16;
+    // address of the operand of column tile g, k-step ks (g, ks: unrolled constants)
+    auto operand = [&](int g, int ks) -> const unsigned char * {
+        if constexpr (NAT == 0) return vb[0] + (ks * G + g) * kLdsBlockBytes;
+        else if constexpr (NAT == 1) return vb[(g & 1) * 2 + ks] + 256 * (g >> 1);
+        else return vb[ks] + 256 * g;
+    };
     const bool ragged_k = (K & 31) != 0;
     const bool k_live = (nks - 1) * 32 + rg * 8 < K;
     // A negative softmax scale is applied as |scale| to negated scores: the sign bits of the A
@@ -493,7 +544,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         f32x4 acc[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + g * kLdsBlockBytes);
+            const u32x4 bf = *reinterpret_cast<const u32x4 *>(operand(g, 0));
             acc[g] = Elem<DT>::mfma(af[0], bf, f32x4{0.f, 0.f, 0.f, 0.f});
         }
 #pragma unroll
@@ -501,7 +552,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
             if (ks < nks) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    const u32x4 bf = *reinterpret_cast<const u32x4 *>(blk + (ks * G + g) * kLdsBlockBytes);
+                    const u32x4 bf = *reinterpret_cast<const u32x4 *>(operand(g, ks));
                     acc[g] = Elem<DT>::mfma(af[ks], bf, acc[g]);
                 }
             }
@@ -529,7 +580,20 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
 template <int DT, bool FUSED, bool F32OUT, int MAXNT>
 __device__ __forceinline__ void strips_exact_dispatch(int tiles, const Seg &s, const RunArgs &a, unsigned char *lds,
                                                       int wave, int first_strip, int strip_step) {
-#define BA_EXACT(G_) case G_: strips_exact<DT, G_, FUSED, F32OUT>(s, a, lds, wave, first_strip, strip_step); break;
+    // The in-memory image serves the fused kernel (measured: config 2 fused 17.0 -> 15.9 us, config 3 72.8 -> 69.0);
+    // the GEMM-only kernel is faster with the operand-order blocks (config 3: 56 us against 79).
+    // Bytes the image takes: whole KiB for the image and for the copy of the last G rows.
+    const int pieces = s.N * (s.K >> 3);
+    const bool image_fits =
+        (((pieces + 63) & ~63) + ((tiles * (s.K >> 3) + 63) & ~63)) * 16 <= a.lds_blocks * kLdsBlockBytes + a.lds_extra;
+#define BA_EXACT(G_)                                                                                              \
+    case G_:                                                                                                      \
+        if (FUSED && s.K == 64 && image_fits)                                                                     \
+            strips_exact<DT, G_, FUSED, F32OUT, FUSED ? 1 : 0>(s, a, lds, wave, first_strip, strip_step);         \
+        else if (FUSED && s.K == 128 && image_fits)                                                               \
+            strips_exact<DT, G_, FUSED, F32OUT, FUSED ? 2 : 0>(s, a, lds, wave, first_strip, strip_step);         \
+        else strips_exact<DT, G_, FUSED, F32OUT, 0>(s, a, lds, wave, first_strip, strip_step);                    \
+        break;
     switch (tiles) {
         BA_EXACT(2) BA_EXACT(4) BA_EXACT(6) BA_EXACT(8)
         default:
@@ -677,7 +741,9 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
         }
         const int64_t tallest = !info ? 0 : pass == 0 ? info->small_max_M : info->max_M;
         const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots, tallest));
-        const size_t lds_bytes = (size_t)fa.lds_blocks * kLdsBlockBytes;
+        // room for the copy of the ragged run behind the image of B_g, while the total stays within 64 KiB
+        fa.lds_extra = fa.lds_blocks * kLdsBlockBytes + kRaggedCopyBytes <= 65536 ? kRaggedCopyBytes : 0;
+        const size_t lds_bytes = (size_t)fa.lds_blocks * kLdsBlockBytes + fa.lds_extra;
         if (lean_pass)
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         else

@@ -143,7 +143,7 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
 #pragma unroll
                 for (int g = 0; g < G; ++g) x[g] = -x[g];
             }
-            softmax_lane_runs<G>(x, w, c);
+            softmax_lane_runs<G, false>(x, w, c);
         } else {
             // dx = scale * (dy - sum(y * dy)) * y; src is the saved forward output here
             f32x4 dy[G];

@@ -281,6 +281,8 @@ __global__ __launch_bounds__(kTileThreads, 2) void tile_kernel(RunArgs a, int zd
             if (!last_slab) continue;
 
             if (FUSED && !second) {
+#pragma unroll
+                for (int rt = 0; rt < kRT; ++rt) settle_mfma(acc[rt]);
                 auto update = [&](auto weighted) {
                     float w[kCT];
 #pragma unroll
