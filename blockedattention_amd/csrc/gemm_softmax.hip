@@ -531,6 +531,9 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
     const uint32_t run_off = (uint32_t)(rg * N + col0) * kOutBytes;
 
     for (int strip = first_strip; strip < strips; strip += strip_step) {
+        // The operands of B_g are the same for every strip; left alone, the compiler keeps all of them in
+        // registers across the loop and spills.  They are cheap to read again: make it.
+        asm volatile("" ::: "memory");
         if (ragged_k) {
 #pragma unroll
             for (int ks = 0; ks < kFastSteps; ++ks)
@@ -580,18 +583,16 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
 template <int DT, bool FUSED, bool F32OUT, int MAXNT>
 __device__ __forceinline__ void strips_exact_dispatch(int tiles, const Seg &s, const RunArgs &a, unsigned char *lds,
                                                       int wave, int first_strip, int strip_step) {
-    // The in-memory image serves the fused kernel (measured: config 2 fused 17.0 -> 15.9 us, config 3 72.8 -> 69.0);
-    // the GEMM-only kernel is faster with the operand-order blocks (config 3: 56 us against 79).
-    // Bytes the image takes: whole KiB for the image and for the copy of the last G rows.
+    // Bytes the in-memory image of B_g takes: whole KiB for the image and for the copy of the last G rows.
     const int pieces = s.N * (s.K >> 3);
     const bool image_fits =
         (((pieces + 63) & ~63) + ((tiles * (s.K >> 3) + 63) & ~63)) * 16 <= a.lds_blocks * kLdsBlockBytes + a.lds_extra;
 #define BA_EXACT(G_)                                                                                              \
     case G_:                                                                                                      \
-        if (FUSED && s.K == 64 && image_fits)                                                                     \
-            strips_exact<DT, G_, FUSED, F32OUT, FUSED ? 1 : 0>(s, a, lds, wave, first_strip, strip_step);         \
-        else if (FUSED && s.K == 128 && image_fits)                                                               \
-            strips_exact<DT, G_, FUSED, F32OUT, FUSED ? 2 : 0>(s, a, lds, wave, first_strip, strip_step);         \
+        if (s.K == 64 && image_fits)                                                                              \
+            strips_exact<DT, G_, FUSED, F32OUT, 1>(s, a, lds, wave, first_strip, strip_step);                     \
+        else if (s.K == 128 && image_fits)                                                                        \
+            strips_exact<DT, G_, FUSED, F32OUT, 2>(s, a, lds, wave, first_strip, strip_step);                     \
         else strips_exact<DT, G_, FUSED, F32OUT, 0>(s, a, lds, wave, first_strip, strip_step);                    \
         break;
     switch (tiles) {
