@@ -78,23 +78,13 @@ __device__ __forceinline__ int softmax_plan_nseg(const SoftmaxArgs &a) {
 
 // ---------------------------------------------------------------- lane runs
 // G consecutive elements of one row from memory into x[g][e] (any element alignment).
-template <int DT, int G>
-__device__ __forceinline__ void load_run(const typename Io<DT>::T *p, f32x4 (&x)[G], int e) {
-    if constexpr (DT == BA_F32) {
-        const float *q = reinterpret_cast<const float *>(p);
-#pragma unroll
-        for (int k = 0; k + 4 <= G; k += 4) {
-            const f32x4 v = *reinterpret_cast<const f32x4_unaligned *>(q + k);
-            x[k][e] = v[0]; x[k + 1][e] = v[1]; x[k + 2][e] = v[2]; x[k + 3][e] = v[3];
-        }
-        if constexpr ((G & 2) != 0) {
-            const f32x2 v = *reinterpret_cast<const f32x2_unaligned *>(q + (G - 2));
-            x[G - 2][e] = v[0]; x[G - 1][e] = v[1];
-        }
-    } else {
-        typedef Io<DT> I;
+// G consecutive elements of one row as they come from memory (any element alignment); unpacked later,
+// so that the loads of a whole strip are in flight together.
+template <int DT, int G> struct RawRun {
+    typedef typename Io<DT>::T T;
+    uint32_t w[G / 2];
+    __device__ __forceinline__ void load(const T *p) {
         const char *q = reinterpret_cast<const char *>(p);
-        uint32_t w[G / 2];
 #pragma unroll
         for (int k = 0; k + 4 <= G / 2; k += 4) {
             const u32x4 v = *reinterpret_cast<const u32x4_unaligned *>(q + 4 * k);
@@ -106,11 +96,36 @@ __device__ __forceinline__ void load_run(const typename Io<DT>::T *p, f32x4 (&x)
             w[kDone] = v[0]; w[kDone + 1] = v[1];
         }
         if constexpr (((G / 2) & 1) != 0) w[G / 2 - 1] = *reinterpret_cast<const u32_unaligned *>(q + 4 * (G / 2 - 1));
-#pragma unroll
-        for (int k = 0; k < G / 2; ++k) { x[2 * k][e] = I::lo(w[k]); x[2 * k + 1][e] = I::hi(w[k]); }
     }
-}
+    __device__ __forceinline__ void unpack(f32x4 (&x)[G], int e) const {
+#pragma unroll
+        for (int k = 0; k < G / 2; ++k) { x[2 * k][e] = Io<DT>::lo(w[k]); x[2 * k + 1][e] = Io<DT>::hi(w[k]); }
+    }
+};
+template <int G> struct RawRun<BA_F32, G> {
+    typedef float T;
+    float w[G];
+    __device__ __forceinline__ void load(const T *q) {
+#pragma unroll
+        for (int k = 0; k + 4 <= G; k += 4) {
+            const f32x4 v = *reinterpret_cast<const f32x4_unaligned *>(q + k);
+            w[k] = v[0]; w[k + 1] = v[1]; w[k + 2] = v[2]; w[k + 3] = v[3];
+        }
+        if constexpr ((G & 2) != 0) {
+            const f32x2 v = *reinterpret_cast<const f32x2_unaligned *>(q + (G - 2));
+            w[G - 2] = v[0]; w[G - 1] = v[1];
+        }
+    }
+    __device__ __forceinline__ void unpack(f32x4 (&x)[G], int e) const {
+#pragma unroll
+        for (int k = 0; k < G; ++k) x[k][e] = w[k];
+    }
+};
 
+// The 16-row strips first, first + step, ... of one segment with 2 <= cols <= 16 * G.  Every lane loads
+// in every step: lanes past the row end hold the run [cols-G, cols) once more (weight 0), rows past the
+// segment's end repeat its last row (computed, not stored), so no load sits behind a branch; the loads
+// of the next strip are issued before the arithmetic of the current one.
 template <int DT, int G, bool BACKWARD>
 __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0, int rows, int cols, int first_strip,
                                              int strip_step) {
@@ -129,16 +144,27 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
     const float sgn = c_signed < 0.f ? -1.f : 1.f;   // forward works on sgn * x so that the multiplier is >= 0
     const float c = c_signed * sgn;
     const int strips = (rows + 15) >> 4;
+    RawRun<DT, G> rx[4], rd[BACKWARD ? 4 : 1];
+    auto issue = [&](int strip) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            // register e of row group rg is row 16*strip + 4*e + rg: an instruction covers four consecutive rows
+            const int64_t row = min(16 * strip + rg + 4 * e, rows - 1);
+            rx[e].load(src + row * cols);
+            if (BACKWARD) rd[BACKWARD ? e : 0].load(aux + row * cols);
+        }
+    };
+    if (first_strip < strips) issue(first_strip);
     for (int strip = first_strip; strip < strips; strip += strip_step) {
-        // register e of row group rg is row 16*strip + 4*e + rg: an instruction covers four consecutive rows
         const int r0 = 16 * strip + rg;
-        f32x4 x[G];
+        f32x4 x[G], dy[BACKWARD ? G : 1];
 #pragma unroll
-        for (int g = 0; g < G; ++g) x[g] = f32x4{-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f} * sgn;   // lowest after the sign flip
-        if (!BACKWARD) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (owner && r0 + 4 * e < rows) load_run<DT, G>(src + (int64_t)(r0 + 4 * e) * cols, x, e);
+        for (int e = 0; e < 4; ++e) {
+            rx[e].unpack(x, e);
+            if constexpr (BACKWARD) rd[e].unpack(dy, e);
+        }
+        if (strip + strip_step < strips) issue(strip + strip_step);
+        if constexpr (!BACKWARD) {
             if (sgn < 0.f) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) x[g] = -x[g];
@@ -146,15 +172,6 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
             softmax_lane_runs<G, false>(x, w, c);
         } else {
             // dx = scale * (dy - sum(y * dy)) * y; src is the saved forward output here
-            f32x4 dy[G];
-#pragma unroll
-            for (int g = 0; g < G; ++g) { x[g] = f32x4{0.f, 0.f, 0.f, 0.f}; dy[g] = x[g]; }
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (owner && r0 + 4 * e < rows) {
-                    load_run<DT, G>(src + (int64_t)(r0 + 4 * e) * cols, x, e);
-                    load_run<DT, G>(aux + (int64_t)(r0 + 4 * e) * cols, dy, e);
-                }
             float dot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int e = 0; e < 4; ++e)
