@@ -1,9 +1,16 @@
 // fp32 varlen GEMM (the reference's generic kernel, csrc/cuda/spBlkGEMM.cu:120-271,
-// for T = float): fp32 multiply-add on the vector ALU, accumulation in k order.
-// A correctness path for fp32 callers; the fp16/bf16 MFMA kernels are the fast path.
+// for T = float): fp32 multiply-add on the vector ALU, accumulation in k order,
+// any shape, offset and layout (transpose flags).  The fp16/bf16 MFMA kernels are
+// the fast path; this one serves fp32 callers such as the reference's own test.
 //
-// One wavefront computes a 16-row piece of one segment; lane l owns columns
-// c0 + l + 64*j, so the stores of one output row are one contiguous run.
+// Workgroup = 64 rows x 64 columns of one segment and head at a time, k in chunks
+// of 64.  A chunk of B_g (64 columns x 64 k) is staged in LDS by the whole
+// workgroup with coalesced loads along the operand's contiguous dimension, stored
+// [column][k] with an odd pitch; each wavefront stages its own 16 rows of A_g
+// [row][k].  In the inner loop a lane owns one column: it reads its B value per k
+// (one LDS word, lanes on consecutive banks) and the sixteen A values of four k at
+// a time as broadcast 16-byte LDS reads, and does 16 multiply-adds per k.  One
+// store instruction writes 64 consecutive elements of an output row.
 #include <algorithm>
 
 #include "ba_device.hpp"
@@ -13,10 +20,18 @@ namespace ba {
 
 constexpr int kF32Threads = 256;
 constexpr int kF32Waves = kF32Threads / 64;
+constexpr int kF32Cols = 64;                         // columns per block = lanes
+constexpr int kF32K = 64;                            // k per chunk
+constexpr int kF32Rows = kStripRows * kF32Waves;     // rows per workgroup round
+constexpr int kF32PitchB = kF32K + 1;                // odd: lanes (columns) fall on consecutive banks
+constexpr int kF32PitchA = kF32K + 4;                // 16-byte rows, staggered banks
 
-// grid (segment, head, z): the wavefronts of the workgroup take the 16-row
-// strips of one segment of one head.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+// grid (segment, head, z): workgroup z takes the 64-row rounds z, z + gridDim.z, ... of its segment.
 __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
+    __shared__ float sB[kF32Cols * kF32PitchB];
+    __shared__ __attribute__((aligned(16))) float sA[kF32Waves][kStripRows * kF32PitchA];
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
     const uint32_t magic = hdr->magic;
     const int nseg = hdr->nseg, pkind = hdr->kind, bad = hdr->bad_segments;
@@ -32,35 +47,84 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
     const SegRec rec = load_rec(pv.recs, g);
     const int M = rec.M, N = rec.N, K = rec.K;
     if (M < 1 || N < 1) return;
-    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6);
     const int lane = lane_id();
     const bool t1 = a.flags & kFlagTranspose1, t2 = a.flags & kFlagTranspose2;
     const int64_t h = blockIdx.y;
     const float *as = reinterpret_cast<const float *>(a.A) + h * a.Dm1 + rec.off1;
     const float *bs = reinterpret_cast<const float *>(a.B) + h * a.Dm2 + rec.off2;
     float *os = reinterpret_cast<float *>(a.out) + h * a.Dout + rec.offO;
-    const int strips = (M + kStripRows - 1) / kStripRows;
-    for (int strip = blockIdx.z * kF32Waves + wave; strip < strips; strip += gridDim.z * kF32Waves) {
-        const int r0 = strip * kStripRows;
-        const int rows = min(kStripRows, M - r0);
-        for (int col = lane; col < N; col += 64) {
+    float *myA = sA[wave];
+    const int nkc = (K + kF32K - 1) / kF32K;
+
+    for (int round = blockIdx.z; round * kF32Rows < M; round += gridDim.z) {
+        const int r0 = round * kF32Rows + wave * kStripRows;          // this wavefront's 16 rows
+        for (int c0 = 0; c0 < N; c0 += kF32Cols) {
             float acc[kStripRows];
 #pragma unroll
             for (int r = 0; r < kStripRows; ++r) acc[r] = 0.f;
-            for (int t = 0; t < K; ++t) {
-                const float bv = t2 ? bs[(int64_t)t * N + col] : bs[(int64_t)col * K + t];
+            for (int kc = 0; kc < std::max(nkc, 1); ++kc) {
+                const int k0 = kc * kF32K;
+                __syncthreads();                                       // the previous chunk is consumed
+                // ---- B chunk: sB[col][k] = B_g[c0 + col][k0 + k], zero outside the segment
+                if (!t2) {
+                    // rows of B_g are contiguous in k: lane = k, each wavefront 16 columns
+                    const int kk = tid & 63, k = k0 + kk, cq = (tid >> 6) * 16;
 #pragma unroll
-                for (int r = 0; r < kStripRows; ++r) {
-                    if (r < rows) {
-                        const int row = r0 + r;
-                        const float av = t1 ? as[(int64_t)t * M + row] : as[(int64_t)row * K + t];
-                        acc[r] = fmaf(av, bv, acc[r]);
+                    for (int i = 0; i < 16; ++i) {
+                        const int col = cq + i;
+                        sB[col * kF32PitchB + kk] = (c0 + col < N && k < K) ? bs[(int64_t)(c0 + col) * K + k] : 0.f;
+                    }
+                } else {
+                    // stored K x N: contiguous in the column
+                    const int col = tid & 63, kq = (tid >> 6) * 16;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int k = k0 + kq + i;
+                        sB[col * kF32PitchB + kq + i] = (c0 + col < N && k < K) ? bs[(int64_t)k * N + c0 + col] : 0.f;
+                    }
+                }
+                // ---- this wavefront's rows of A: myA[row][k] = A_g[r0 + row][k0 + k]
+                if (!t1) {
+                    // lane = k, one row per step
+#pragma unroll
+                    for (int r = 0; r < kStripRows; ++r) {
+                        const int k = k0 + lane;
+                        myA[r * kF32PitchA + lane] = (r0 + r < M && k < K) ? as[(int64_t)(r0 + r) * K + k] : 0.f;
+                    }
+                } else {
+                    // stored K x M: contiguous in the row index; lane = (k quarter, row)
+                    const int r = lane & 15, kq = lane >> 4;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int kk = kq * 16 + i, k = k0 + kk;
+                        myA[r * kF32PitchA + kk] = (r0 + r < M && k < K) ? as[(int64_t)k * M + r0 + r] : 0.f;
+                    }
+                }
+                __syncthreads();
+                // ---- 64 k of multiply-adds: four k per step
+                const float *bcol = sB + lane * kF32PitchB;
+#pragma unroll 4
+                for (int k4 = 0; k4 < kF32K; k4 += 4) {
+                    f32x4v av[kStripRows];
+#pragma unroll
+                    for (int r = 0; r < kStripRows; ++r)
+                        av[r] = *reinterpret_cast<const f32x4v *>(&myA[r * kF32PitchA + k4]);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const float bv = bcol[k4 + t];
+#pragma unroll
+                        for (int r = 0; r < kStripRows; ++r) acc[r] = fmaf(av[r][t], bv, acc[r]);
                     }
                 }
             }
+            const int col = c0 + lane;
+            if (col < N) {
 #pragma unroll
-            for (int r = 0; r < kStripRows; ++r)
-                if (r < rows) os[(int64_t)(r0 + r) * N + col] = acc[r];
+                for (int r = 0; r < kStripRows; ++r)
+                    if (r0 + r < M) os[(int64_t)(r0 + r) * N + col] = acc[r];
+            }
         }
     }
 }
@@ -70,7 +134,9 @@ int launch_gemm_f32(const RunArgs &args, int64_t nseg, const ba_plan_info *info,
     int64_t z = 4;
     if (info) {
         nseg = info->nseg;
-        z = std::max<int64_t>(1, std::min<int64_t>(64, (info->max_M + kStripRows * kF32Waves - 1) / (kStripRows * kF32Waves)));
+        const int64_t rounds = (std::max<int64_t>(info->max_M, 1) + kF32Rows - 1) / kF32Rows;
+        const int64_t want = ((int64_t)device_cu_count() * 8 + nseg * args.H - 1) / std::max<int64_t>(1, nseg * args.H);
+        z = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(rounds, want), 64));
     }
     if (nseg <= 0) return BA_OK;
     hipLaunchKernelGGL(gemm_f32_kernel, dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z), dim3(kF32Threads), 0,
