@@ -1,16 +1,15 @@
 // fp32 varlen GEMM (the reference's generic kernel, csrc/cuda/spBlkGEMM.cu:120-271,
-// for T = float): fp32 multiply-add on the vector ALU, accumulation in k order,
-// any shape, offset and layout (transpose flags).  The fp16/bf16 MFMA kernels are
-// the fast path; this one serves fp32 callers such as the reference's own test.
+// for T = float) on the fp32 matrix instruction (v_mfma_f32_16x16x4_f32, fp32
+// products and sums), any shape, offset and layout (transpose flags).  It serves
+// fp32 callers such as the reference's own test; fp16/bf16 have their own kernels.
 //
 // Workgroup = 64 rows x 64 columns of one segment and head at a time, k in chunks
 // of 64.  A chunk of B_g (64 columns x 64 k) is staged in LDS by the whole
 // workgroup with coalesced loads along the operand's contiguous dimension, stored
 // [column][k] with an odd pitch; each wavefront stages its own 16 rows of A_g
-// [row][k].  In the inner loop a lane owns one column: it reads its B value per k
-// (one LDS word, lanes on consecutive banks) and the sixteen A values of four k at
-// a time as broadcast 16-byte LDS reads, and does 16 multiply-adds per k.  One
-// store instruction writes 64 consecutive elements of an output row.
+// [row][k].  A wavefront computes 16 rows x 64 columns as four 16 x 16 tiles: per
+// four k it reads one A word and four B words per lane from LDS and issues four
+// matrix instructions.
 #include <algorithm>
 
 #include "ba_device.hpp"
@@ -61,9 +60,10 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
     for (int round = blockIdx.z; round * kF32Rows < M; round += gridDim.z) {
         const int r0 = round * kF32Rows + wave * kStripRows;          // this wavefront's 16 rows
         for (int c0 = 0; c0 < N; c0 += kF32Cols) {
-            float acc[kStripRows];
+            // four 16 x 16 tiles per wavefront: lane (j = lane%16, q = lane/16) holds rows 4q..4q+3 of column j
+            f32x4v acc[kF32Cols / 16];
 #pragma unroll
-            for (int r = 0; r < kStripRows; ++r) acc[r] = 0.f;
+            for (int t = 0; t < kF32Cols / 16; ++t) acc[t] = f32x4v{0.f, 0.f, 0.f, 0.f};
             for (int kc = 0; kc < std::max(nkc, 1); ++kc) {
                 const int k0 = kc * kF32K;
                 __syncthreads();                                       // the previous chunk is consumed
@@ -103,27 +103,27 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
                     }
                 }
                 __syncthreads();
-                // ---- 64 k of multiply-adds: four k per step
-                const float *bcol = sB + lane * kF32PitchB;
+                // ---- 64 k on the matrix unit, four k per instruction (v_mfma_f32_16x16x4_f32):
+                //      operand lane (i = lane%16, q = lane/16) supplies row / column i at k + q
+                const float *arow = myA + (lane & 15) * kF32PitchA + (lane >> 4);
+                const float *bcol = sB + (lane & 15) * kF32PitchB + (lane >> 4);
 #pragma unroll 4
                 for (int k4 = 0; k4 < kF32K; k4 += 4) {
-                    f32x4v av[kStripRows];
+                    const float av = arow[k4];
 #pragma unroll
-                    for (int r = 0; r < kStripRows; ++r)
-                        av[r] = *reinterpret_cast<const f32x4v *>(&myA[r * kF32PitchA + k4]);
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const float bv = bcol[k4 + t];
-#pragma unroll
-                        for (int r = 0; r < kStripRows; ++r) acc[r] = fmaf(av[r][t], bv, acc[r]);
-                    }
+                    for (int t = 0; t < kF32Cols / 16; ++t)
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bcol[t * 16 * kF32PitchB + k4], acc[t], 0, 0, 0);
                 }
             }
-            const int col = c0 + lane;
-            if (col < N) {
+            const int j = lane & 15, q = lane >> 4;
 #pragma unroll
-                for (int r = 0; r < kStripRows; ++r)
-                    if (r0 + r < M) os[(int64_t)(r0 + r) * N + col] = acc[r];
+            for (int t = 0; t < kF32Cols / 16; ++t) {
+                const int col = c0 + 16 * t + j;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = r0 + 4 * q + e;
+                    if (col < N && row < M) os[(int64_t)row * N + col] = acc[t][e];
+                }
             }
         }
     }
