@@ -265,6 +265,14 @@ def main():
         blockedAttention.set_schedule_cache(8)
     except ImportError as e:
         line["detail"]["torch_op_us"] = f"extension not built: {e}"
+    # context for the roofline fraction: what a plain device-to-device copy of 512 MiB sustains on this box
+    # (bytes read + bytes written per second), i.e. the rate a perfectly streaming kernel reaches
+    import torch
+    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    copy_us = case.event_us(lambda: dst.copy_(src), 10, 2)
+    line["detail"]["device_copy_GBps"] = round(2 * src.numel() / copy_us * 1e-3, 1)
+    del src, dst
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(case, args.cpu_seconds)
     if not args.no_others:
