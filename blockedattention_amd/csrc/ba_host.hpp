@@ -13,6 +13,7 @@ enum RunFlags : int {
     kFlagTranspose2 = 2,   // B segments stored K x N
     kFlagMfmaOk = 4,       // layouts, base pointers and head strides allow 16-byte operand loads
     kFlagOutF32 = 8,       // fused path writes fp32 probabilities
+    kFlagPacksToo = 16,    // strip kernel: the blocks behind its own list walk the pack leaders of the rest list
     kFlagQuiet = 64        // an earlier launch of the same call reports a plan that does not match
 };
 

@@ -680,7 +680,19 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
         if (!(a.flags & kFlagQuiet)) report_mismatch(a);
         return;
     }
-    if (!valid) return;
+    if (!valid) {
+        // Blocks behind the kernel's own list: with kFlagPacksToo they take the packs of tiny segments
+        // (the rest list then holds nothing but pack leaders), which saves the call a launch.
+        if (a.flags & kFlagPacksToo) {
+            const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+            const int slot = (int)blockIdx.x - (int)hdr->totals[a.list], packs = (int)hdr->totals[kListRest];
+            if (slot >= 0 && slot < packs && blockIdx.z == 0 && threadIdx.x < 64) {
+                const SegRec r = load_rec(pv.recs + (int64_t)(kListRest + 1) * plan_cap(a.nseg), slot);
+                if (r.kind == kSegPackLead) wave_pack<DT, FUSED, F32OUT>(pv, r.index, r.packLen, h, a);
+            }
+        }
+        return;
+    }
     const int tiles = fast_strip_tiles(s.N);
     const int need = strip_blocks(s.N, s.K);
     // the lists hold only segments of this kernel; the checks guard against a launch that does not match
@@ -726,10 +738,19 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
         const int64_t want = ceil_div((int64_t)cus * 8, std::max<int64_t>(1, slots * (int64_t)H));
         return std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
     };
+    // the rest list is nothing but pack leaders: the first strip launch takes them along
+    const bool packs_ride = info && mfma_ok && n_rest > 0 && n_rest == info->pack_items && info->slow_items == 0 &&
+                            (n_small > 0 || n_big > 0);
+    bool packs_taken = false;
     for (int pass = 0; pass < 2; ++pass) {
-        const int64_t slots = pass == 0 ? n_small : n_big;
+        int64_t slots = pass == 0 ? n_small : n_big;
         if (slots <= 0) continue;
         RunArgs fa = args;
+        if (packs_ride && !packs_taken) {
+            fa.flags |= kFlagPacksToo;
+            slots += n_rest;
+            packs_taken = true;
+        }
         fa.list = pass == 0 ? kListSmall : kListBig;
         fa.lds_blocks = pass == 0 ? kFastBlocks : kBigBlocks;
         bool lean_pass = lean;
@@ -758,7 +779,7 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
         if (st != BA_OK) return st;
         args.flags |= kFlagQuiet;
     }
-    if (n_rest > 0) {
+    if (n_rest > 0 && !packs_taken) {
         // z spreads the 16-row strips (or rows) of the largest segment over workgroups
         int64_t z = 4, blocks = 32;
         if (info) {
