@@ -14,6 +14,7 @@ enum RunFlags : int {
     kFlagMfmaOk = 4,       // layouts, base pointers and head strides allow 16-byte operand loads
     kFlagOutF32 = 8,       // fused path writes fp32 probabilities
     kFlagPacksToo = 16,    // strip kernel: the blocks behind its own list walk the pack leaders of the rest list
+    kFlagTilesToo = 32,    // strip kernel, 64 KiB launch: further blocks run the tile kernel's workgroups (tile_zdim, tile_groups)
     kFlagQuiet = 64        // an earlier launch of the same call reports a plan that does not match
 };
 
@@ -29,6 +30,10 @@ struct RunArgs {
     int list;         // work list the launch walks (PrefixKind), or -1: every segment, by block index
     int nseg;         // segment count the plan was built for (checked against the plan)
     int lds_extra;    // bytes of dynamic LDS behind the operand blocks (strip kernel: copy of the ragged run)
+    int tile_zdim;    // with kFlagTilesToo: row-block dimension and number of workgroups of the tile kernel,
+    int tile_groups;  // which take the first tile_groups blocks of a flat grid; the strip part then has
+    int ride_slots;   // ride_slots x H x ride_z workgroups, slot fastest
+    int ride_z;
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,

@@ -20,6 +20,7 @@
 #include <algorithm>
 
 #include "ba_gemm_common.hpp"
+#include "tile_body.hpp"
 
 namespace ba {
 
@@ -667,15 +668,33 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 6 : 4) void segment_kerne
 // strip_kernel: the strip-class segments whose B_g fits the LDS window, nothing else.
 // Grid (segment, head, z); the workgroups with the same (segment, head) share the
 // segment's strips round-robin.
-template <int DT, bool FUSED, bool F32OUT, int MAXNT>
+// RIDE: the build whose launch also carries the tile kernel's workgroups.  Its grid is flat: the first
+// a.tile_groups blocks are tile workgroups (they run longest, so they start first), the rest decode to
+// (slot, head, z) with the slot fastest.  Two launches that each fill half the machine become one.
+template <int DT, bool FUSED, bool F32OUT, int MAXNT, bool RIDE = false>
 __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(RunArgs a) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    unsigned bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z, gz = gridDim.z;
+    if constexpr (RIDE) {
+        if (bx < (unsigned)a.tile_groups) {
+            RunArgs ta = a;
+            ta.list = kListTile;
+            ta.flags |= kFlagQuiet;
+            tile_block<DT, FUSED, F32OUT>(ta, a.tile_zdim, bx, lds);
+            return;
+        }
+        const unsigned lin = bx - (unsigned)a.tile_groups;
+        bx = lin % (unsigned)a.ride_slots;
+        by = (lin / (unsigned)a.ride_slots) % (unsigned)a.H;
+        bz = lin / ((unsigned)a.ride_slots * (unsigned)a.H);
+        gz = (unsigned)a.ride_z;
+    }
     const PlanRO pv = plan_ro(a.plan, a.nseg);
-    const int64_t h = blockIdx.y;
+    const int64_t h = by;
     // header and record are fetched together; nothing waits on the header alone
     const bool ok = header_ok(a);
     bool valid;
-    const Seg s = load_listed(pv, blockIdx.x, h, a, valid);
+    const Seg s = load_listed(pv, bx, h, a, valid);
     if (!ok) {
         if (!(a.flags & kFlagQuiet)) report_mismatch(a);
         return;
@@ -685,8 +704,8 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
         // (the rest list then holds nothing but pack leaders), which saves the call a launch.
         if (a.flags & kFlagPacksToo) {
             const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
-            const int slot = (int)blockIdx.x - (int)hdr->totals[a.list], packs = (int)hdr->totals[kListRest];
-            if (slot >= 0 && slot < packs && blockIdx.z == 0 && threadIdx.x < 64) {
+            const int slot = (int)bx - (int)hdr->totals[a.list], packs = (int)hdr->totals[kListRest];
+            if (slot >= 0 && slot < packs && bz == 0 && threadIdx.x < 64) {
                 const SegRec r = load_rec(pv.recs + (int64_t)(kListRest + 1) * plan_cap(a.nseg), slot);
                 if (r.kind == kSegPackLead) wave_pack<DT, FUSED, F32OUT>(pv, r.index, r.packLen, h, a);
             }
@@ -698,8 +717,8 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
     // the lists hold only segments of this kernel; the checks guard against a launch that does not match
     if ((s.kind != kSegStrip) | (need < 1) | (need > a.lds_blocks) | (tiles > MAXNT)) return;
     const int wave = uniform((int)(threadIdx.x >> 6));
-    const int first = blockIdx.z * kSegWaves + wave, step = gridDim.z * kSegWaves;
-    if ((int)blockIdx.z * kSegWaves * kStripRows >= s.M) return;   // no strip for this workgroup
+    const int first = bz * kSegWaves + wave, step = gz * kSegWaves;
+    if ((int)bz * kSegWaves * kStripRows >= s.M) return;   // no strip for this workgroup
     strips_exact_dispatch<DT, FUSED, F32OUT, MAXNT>(tiles, s, a, lds, wave, first, step);
 }
 
@@ -742,6 +761,12 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     const bool packs_ride = info && mfma_ok && n_rest > 0 && n_rest == info->pack_items && info->slow_items == 0 &&
                             (n_small > 0 || n_big > 0);
     bool packs_taken = false;
+    // a modest amount of tile-kernel work rides in the strip kernel's 64 KiB launch (same LDS, same
+    // residency) instead of following it; large tile work keeps its own die-aware launch
+    const int64_t tile_z = !info ? 1 : std::max<int64_t>(1, std::min<int64_t>(64, ceil_div(std::max<int64_t>(info->max_M, 1), kTileRows)));
+    const int64_t tile_groups = ceil_div(n_tile, kDies) * kDies * (int64_t)H * tile_z;
+    const bool tiles_ride = info && n_big > 0 && n_tile > 0 && tile_groups <= 4096 && (dtype == BA_F16 || dtype == BA_BF16);
+    bool tiles_taken = false;
     for (int pass = 0; pass < 2; ++pass) {
         int64_t slots = pass == 0 ? n_small : n_big;
         if (slots <= 0) continue;
@@ -750,6 +775,15 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
             fa.flags |= kFlagPacksToo;
             slots += n_rest;
             packs_taken = true;
+        }
+        const bool ride = pass == 1 && tiles_ride;
+        if (ride) {
+            fa.flags |= kFlagTilesToo;
+            fa.tile_zdim = (int)tile_z;
+            fa.tile_groups = (int)tile_groups;
+            fa.ride_slots = (int)slots;
+            fa.ride_z = (int)strip_z(slots, info->max_M);
+            tiles_taken = true;
         }
         fa.list = pass == 0 ? kListSmall : kListBig;
         fa.lds_blocks = pass == 0 ? kFastBlocks : kBigBlocks;
@@ -766,13 +800,17 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
         // room for the copy of the ragged run behind the image of B_g, while the total stays within 64 KiB
         fa.lds_extra = fa.lds_blocks * kLdsBlockBytes + kRaggedCopyBytes <= 65536 ? kRaggedCopyBytes : 0;
         const size_t lds_bytes = (size_t)fa.lds_blocks * kLdsBlockBytes + fa.lds_extra;
-        if (lean_pass)
+        if (ride)
+            hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 16, true>),
+                               dim3((unsigned)(tile_groups + slots * (int64_t)H * fa.ride_z)), dim3(kSegThreads), lds_bytes,
+                               stream, fa);
+        else if (lean_pass)
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 8>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         else
             hipLaunchKernelGGL((strip_kernel<DT, FUSED, F32OUT, 16>), grid, dim3(kSegThreads), lds_bytes, stream, fa);
         args.flags |= kFlagQuiet;
     }
-    if (n_tile > 0) {
+    if (n_tile > 0 && !tiles_taken) {
         RunArgs ta = args;
         ta.list = kListTile;
         const int st = launch_tiles(dtype, FUSED ? 1 : 0, ta, n_tile, info, stream);
