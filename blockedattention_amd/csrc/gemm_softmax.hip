@@ -733,8 +733,11 @@ static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 //                   second launch: up to 64 KiB, fewer resident workgroups)
 //   tile kernel     large segments (see tile_segment())
 //   segment kernel  packs, the element-wise class, and what the others leave
-// With a host copy of the plan summary the grids are exactly the list lengths and empty lists are not
-// launched; without it every kernel is launched over nseg slots and reads its list length from the plan.
+// With a host copy of the plan summary the grids are exactly the list lengths, empty lists are not
+// launched, and launches are merged where that saves one: the packs ride in the first strip launch
+// when the rest list holds nothing else, and a modest amount of tile-kernel work rides in the 64 KiB
+// strip launch.  Without the summary every kernel is launched over nseg slots and reads its list
+// length from the plan.
 // The first launch reports a plan that does not match the call; the later ones stay quiet.
 template <int DT, bool FUSED, bool F32OUT>
 static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
