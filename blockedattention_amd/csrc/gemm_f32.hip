@@ -64,42 +64,53 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
             f32x4v acc[kF32Cols / 16];
 #pragma unroll
             for (int t = 0; t < kF32Cols / 16; ++t) acc[t] = f32x4v{0.f, 0.f, 0.f, 0.f};
-            for (int kc = 0; kc < std::max(nkc, 1); ++kc) {
+            for (int kc = 0; kc < nkc; ++kc) {                         // K = 0: no chunk, the result is zeros
                 const int k0 = kc * kF32K;
                 __syncthreads();                                       // the previous chunk is consumed
+                // Staging: every load is unconditional (index clamped into the segment, value zeroed
+                // afterwards where it lies outside), so the sixteen loads of a thread are in flight together.
                 // ---- B chunk: sB[col][k] = B_g[c0 + col][k0 + k], zero outside the segment
-                if (!t2) {
-                    // rows of B_g are contiguous in k: lane = k, each wavefront 16 columns
-                    const int kk = tid & 63, k = k0 + kk, cq = (tid >> 6) * 16;
+                {
+                    float v[16];
+                    if (!t2) {
+                        // rows of B_g are contiguous in k: lane = k, each wavefront 16 columns
+                        const int kk = tid & 63, k = k0 + kk, cq = (tid >> 6) * 16;
+                        const int kc_ = min(k, K - 1);
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int col = cq + i;
-                        sB[col * kF32PitchB + kk] = (c0 + col < N && k < K) ? bs[(int64_t)(c0 + col) * K + k] : 0.f;
-                    }
-                } else {
-                    // stored K x N: contiguous in the column
-                    const int col = tid & 63, kq = (tid >> 6) * 16;
+                        for (int i = 0; i < 16; ++i) v[i] = bs[(int64_t)min(c0 + cq + i, N - 1) * K + kc_];
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int k = k0 + kq + i;
-                        sB[col * kF32PitchB + kq + i] = (c0 + col < N && k < K) ? bs[(int64_t)k * N + c0 + col] : 0.f;
+                        for (int i = 0; i < 16; ++i)
+                            sB[(cq + i) * kF32PitchB + kk] = (c0 + cq + i < N && k < K) ? v[i] : 0.f;
+                    } else {
+                        // stored K x N: contiguous in the column
+                        const int col = tid & 63, kq = (tid >> 6) * 16;
+                        const int cc = min(c0 + col, N - 1);
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) v[i] = bs[(int64_t)min(k0 + kq + i, K - 1) * N + cc];
+#pragma unroll
+                        for (int i = 0; i < 16; ++i)
+                            sB[col * kF32PitchB + kq + i] = (c0 + col < N && k0 + kq + i < K) ? v[i] : 0.f;
                     }
                 }
                 // ---- this wavefront's rows of A: myA[row][k] = A_g[r0 + row][k0 + k]
-                if (!t1) {
-                    // lane = k, one row per step
+                {
+                    float v[16];
+                    if (!t1) {
+                        // lane = k, one row per step
+                        const int k = k0 + lane, kc_ = min(k, K - 1);
 #pragma unroll
-                    for (int r = 0; r < kStripRows; ++r) {
-                        const int k = k0 + lane;
-                        myA[r * kF32PitchA + lane] = (r0 + r < M && k < K) ? as[(int64_t)(r0 + r) * K + k] : 0.f;
-                    }
-                } else {
-                    // stored K x M: contiguous in the row index; lane = (k quarter, row)
-                    const int r = lane & 15, kq = lane >> 4;
+                        for (int r = 0; r < kStripRows; ++r) v[r] = as[(int64_t)min(r0 + r, M - 1) * K + kc_];
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int kk = kq * 16 + i, k = k0 + kk;
-                        myA[r * kF32PitchA + kk] = (r0 + r < M && k < K) ? as[(int64_t)k * M + r0 + r] : 0.f;
+                        for (int r = 0; r < kStripRows; ++r)
+                            myA[r * kF32PitchA + lane] = (r0 + r < M && k < K) ? v[r] : 0.f;
+                    } else {
+                        // stored K x M: contiguous in the row index; lane = (k quarter, row)
+                        const int r = lane & 15, kq = lane >> 4, rc = min(r0 + r, M - 1);
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) v[i] = as[(int64_t)min(k0 + kq * 16 + i, K - 1) * M + rc];
+#pragma unroll
+                        for (int i = 0; i < 16; ++i)
+                            myA[r * kF32PitchA + kq * 16 + i] = (r0 + r < M && k0 + kq * 16 + i < K) ? v[i] : 0.f;
                     }
                 }
                 __syncthreads();
