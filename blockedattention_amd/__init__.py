@@ -1,12 +1,13 @@
 """MI355X-native varlen ("blocked") GEMM and blocked row softmax.
 
 ``blockGEMM`` / ``blockSoftmax`` keep the reference package's signatures;
-``blockGEMMSoftmax`` is the fused pair.  ``capi`` exposes the C ABI directly.
+``blockGEMMSoftmax`` is the fused pair, ``blockFusedAttention`` the one-pass
+``softmax(scale q k^T) v``.  ``capi`` exposes the C ABI directly.
 Importing the operators needs the in-tree build (``python -m
 blockedattention_amd.build``); nothing falls back to PyTorch or the CPU.
 """
 
-__all__ = ["blockGEMM", "blockSoftmax", "blockGEMMSoftmax", "set_schedule_cache", "schedule_cache_stats"]
+__all__ = ["blockGEMM", "blockSoftmax", "blockGEMMSoftmax", "blockFusedAttention", "set_schedule_cache", "schedule_cache_stats"]
 
 
 def __getattr__(name):

@@ -70,6 +70,25 @@ def blockGEMMSoftmax(
                                                    float(scale), bool(out_fp32))
 
 
+def blockFusedAttention(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+    MList: Optional[torch.Tensor] = None, NList: Optional[torch.Tensor] = None, KList: Optional[torch.Tensor] = None,
+    mat1Accum: Optional[torch.Tensor] = None, mat2Accum: Optional[torch.Tensor] = None,
+    outAccum: Optional[torch.Tensor] = None,
+    scale: float = 1.0,
+) -> torch.Tensor:
+    """``softmax(scale * Q_g @ K_g^T) @ V_g`` per segment in one pass (forward only).
+
+    ``q`` is ``[H, sum(M*K)]`` (the first operand of ``blockGEMM``), ``k`` and ``v`` are both
+    ``[H, sum(N*K)]`` (its second operand's layout); the metadata is ``blockGEMM``'s.  The result,
+    ``[H, sum(M*K)]``, is what ``blockGEMM(blockSoftmax(blockGEMM(q, k, ...), M, N, scale=scale), v, ...,
+    transpose2=True)`` computes, without the ``M x N`` arrays ever reaching memory.  Head dimensions up
+    to 128.
+    """
+    return blockAttention.sparseBlockedAttention(q, k, v, mat1Accum, mat2Accum, outAccum, MList, NList, KList,
+                                                 float(scale))
+
+
 def set_schedule_cache(capacity: int) -> None:
     """How many schedules the operators keep for metadata tensors they have seen (default 8; 0 = off).
 

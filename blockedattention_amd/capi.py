@@ -18,6 +18,7 @@ META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
 SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
     "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax", "ba_repack_operand",
+    "ba_varlen_attention",
 )
 
 
@@ -77,6 +78,8 @@ def load():
     lib.ba_repack_operand.argtypes = [vp, i32, i32, i32, vp, i32, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, i64, i64, i64, vp]
     lib.ba_gemm_softmax.restype = i32
     lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
+    lib.ba_varlen_attention.restype = i32
+    lib.ba_varlen_attention.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, vp, i64, i64, i64, i64, f32, vp]
     _lib = lib
     return lib
 
@@ -194,6 +197,14 @@ def gemm_softmax(plan, A, B, out, H, Dm1, Dm2, Dout, scale=1.0):
     st = load().ba_gemm_softmax(plan.ptr, plan._hint(), plan.nseg, dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out),
                                 dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
     check(st, "ba_gemm_softmax")
+    return out
+
+
+def varlen_attention(plan, Q, K, V, out, H, Dm1, Dm2, Dout, scale=1.0):
+    """out [H, Dm1] <- softmax(scale * Q_g K_g^T) V_g per segment (see ba_varlen_attention)."""
+    st = load().ba_varlen_attention(plan.ptr, plan._hint(), plan.nseg, dtype_code(Q.dtype), _ptr(Q), _ptr(K), _ptr(V),
+                                    _ptr(out), H, Dm1, Dm2, Dout, float(scale), _stream())
+    check(st, "ba_varlen_attention")
     return out
 
 

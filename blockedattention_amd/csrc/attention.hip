@@ -1,0 +1,380 @@
+// Varlen attention in one pass: O_g = softmax(scale * Q_g K_g^T) V_g per segment and head, with the
+// probabilities never written to memory.  It is what a caller of the reference gets from
+// blockGEMM -> blockSoftmax -> blockGEMM (README.md:3; csrc/sparseBlockedAttention.cpp:118-131) when
+// the probabilities themselves are not wanted: the M x N array, which bounds every other kernel of
+// this library, stays in registers.
+//
+// Layout: Q_g is the M x K operand of the plan (offset off1), K_g and V_g are N x K (offset off2,
+// both with the per-head stride Dm2), O_g is M x K at off1 of a [H, Dm1] buffer.  K <= 128.
+//
+// Workgroup = 4 wavefronts = 64 queries of one segment and head; the keys go by in blocks of 64.
+// Per block the workgroup stages K_g's rows (as they lie, zero padded to a multiple of 32 in k) and
+// V_g's rows TRANSPOSED (one LDS row per output column, keys along the row) in LDS.  A wavefront owns
+// 16 queries:
+//   S^T block  = K_blk Q^T   (matrix instructions, A operand = key rows from LDS, B operand = the
+//                wavefront's query rows, held in registers for the whole pass); the lane
+//                (j = lane%16, rg = lane/16) then holds query j's scores for keys 16t + 4rg + e;
+//   online softmax: running row maximum m and row sum l per query (per lane; the four lanes of a
+//                query exchange the block maximum), accumulators rescaled by 2^((m_old - m_new) c);
+//   O^T       += V_blk^T P^T (A operand = transposed value rows from LDS, B operand = the lane's own
+//                probabilities rounded to the 16-bit type: the k index of the instruction runs over
+//                keys in the order the score registers hold them, so P never moves between lanes).
+// The query index is lane%16 in scores and outputs alike, so m, l and the rescaling are per lane.
+#include <stdlib.h>
+
+#include <algorithm>
+
+#include "ba_device.hpp"
+#include "ba_gemm_common.hpp"
+#include "ba_host.hpp"
+
+namespace ba {
+
+constexpr int kAttThreads = 256;
+constexpr int kAttWaves = kAttThreads / 64;
+constexpr int kAttKeys = 64;                          // keys per block
+constexpr int kAttRows = 16 * kAttWaves;              // queries per workgroup round
+constexpr int kAttPitchV = kAttKeys * 2 + 8;          // bytes per LDS row of transposed values.  An LDS access
+// serves 16 lanes x 8 bytes at a time; the 8-byte skew puts the sixteen rows 16 t + j that an operand read
+// touches in sixteen different 8-byte bank groups, and a staging write covers one row's 128 bytes.
+
+// Eight consecutive elements k0 .. k0+7 of a row of K elements, zeros at and past K, for rows whose
+// length is not a multiple of 8 (pieces straddle nothing, but the row may end inside one): element by
+// element, one load in flight, few registers -- the slow path must not set the register count of the
+// kernel.  Each step shifts the 128-bit value down by one element and puts the new one on top.
+__device__ __forceinline__ u32x4 load8_slow(const uint16_t *row, int k0, int K) {
+    uint32_t r0 = 0, r1 = 0, r2 = 0, r3 = 0;
+#pragma nounroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t x = row[min(k0 + i, K - 1)];
+        r0 = (r0 >> 16) | (r1 << 16);
+        r1 = (r1 >> 16) | (r2 << 16);
+        r2 = (r2 >> 16) | (r3 << 16);
+        r3 = (r3 >> 16) | ((k0 + i < K ? x : 0u) << 16);
+    }
+    return u32x4{r0, r1, r2, r3};
+}
+
+// NK = 32-wide k steps (head dimension padded to 32 * NK).  VEC: the segment's K is a multiple of 8, its
+// rows come as 16-byte loads; otherwise element by element.  The two are separate instances of the whole
+// body so that the slow loads do not sit inside the fast path's loops.
+template <int DT, int NK, int QT, bool VEC>
+__device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbuf, const SegRec &rec, unsigned char *sK,
+                                               unsigned char *sV) {
+    constexpr int KP = 32 * NK;                       // padded head dimension
+    constexpr int kPitchK = KP * 2 + 16;              // bytes per LDS row of keys (16-byte skew: 16 lanes of
+                                                      // a 16-byte read cover all banks once)
+    constexpr int kPieces = KP / 8;                   // 16-byte pieces per row
+    constexpr int kOutTiles = KP / 16;
+    const int M = rec.M, N = rec.N, K = rec.K;
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6);
+    const int lane = lane_id();
+    const int j = lane & 15, rg = lane >> 4;
+    const int64_t h = blockIdx.y;
+    const uint16_t *qs = reinterpret_cast<const uint16_t *>(a.A) + h * a.Dm1 + rec.off1;
+    const uint16_t *ks = reinterpret_cast<const uint16_t *>(a.B) + h * a.Dm2 + rec.off2;
+    const uint16_t *vs = reinterpret_cast<const uint16_t *>(Vbuf) + h * a.Dm2 + rec.off2;
+    uint16_t *os = reinterpret_cast<uint16_t *>(a.out) + h * a.Dm1 + rec.off1;
+
+    // A negative scale is applied as |scale| to negated scores (sign bits of the query operand flipped),
+    // so that the running maximum is always the value to subtract.
+    const float c_signed = a.scale * kLog2e;
+    const float c = __builtin_fabsf(c_signed);
+    const uint32_t flip = c_signed < 0.f ? 0x80008000u : 0u;
+    const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
+
+    // Staging, per thread: NK 16-byte pieces of the key rows (piece u = step * 256 + tid: row u / kPieces,
+    // column 8 * (u % kPieces)) and 4 keys x 8 columns of values (key group tid % 16, piece tid / 16; a load
+    // instruction of a wavefront then covers 64 contiguous bytes of sixteen rows, a write 128 of one).  Element
+    // offsets inside a segment fit 32 bits (checked by the kernel).
+    const int v_kg = tid & 15, v_piece = tid >> 4;    // sixteen lanes = the sixteen key groups of one piece
+    const bool v_thread = v_piece < kPieces;
+    uint32_t k_col[NK], k_off[NK];
+#pragma unroll
+    for (int step = 0; step < NK; ++step) {
+        const int u = step * kAttThreads + tid;
+        k_col[step] = (uint32_t)max(min(8 * (u % kPieces), K - 8), 0);
+        k_off[step] = (uint32_t)(u / kPieces) * (uint32_t)K + k_col[step];
+    }
+    const uint32_t v_col = (uint32_t)max(min(8 * v_piece, K - 8), 0);
+    const uint32_t v_off = (uint32_t)(4 * v_kg) * (uint32_t)K + v_col;
+
+    constexpr int kRoundRows = kAttRows * QT;           // queries per workgroup round
+    for (int round = blockIdx.z; round * kRoundRows < M; round += gridDim.z) {
+        // strip q of the wavefront: rows round * kRoundRows + 64 q + 16 wave ..; the live ones come first
+        const int r0 = round * kRoundRows + wave * 16;
+        const int nq = uniform(r0 >= M ? 0 : min(QT, (M - r0 + kAttRows - 1) / kAttRows));   // 0: the wavefront only stages
+        // the wavefront's queries as B operand: lane (query j, rg) holds k = 32 s + 8 rg .. + 7
+        u32x4 qf[QT][NK];
+#pragma unroll
+        for (int q = 0; q < QT; ++q) {
+            const uint16_t *qrow = qs + (int64_t)min(r0 + kAttRows * q + j, M - 1) * K;
+            if constexpr (VEC) {
+#pragma unroll
+                for (int s = 0; s < NK; ++s)
+                    qf[q][s] = *reinterpret_cast<const u32x4_unaligned *>(qrow + min(32 * s + 8 * rg, K - 8));
+            } else {
+#pragma unroll
+                for (int s = 0; s < NK; ++s) qf[q][s] = load8_slow(qrow, 32 * s + 8 * rg, K);
+            }
+#pragma unroll
+            for (int s = 0; s < NK; ++s) {
+                qf[q][s] = 32 * s + 8 * rg < K ? qf[q][s] : zero4;
+                qf[q][s] = u32x4{qf[q][s][0] ^ flip, qf[q][s][1] ^ flip, qf[q][s][2] ^ flip, qf[q][s][3] ^ flip};
+            }
+        }
+        float m[QT], lsum[QT];
+        f32x4 oacc[QT][kOutTiles];
+#pragma unroll
+        for (int q = 0; q < QT; ++q) {
+            m[q] = -INFINITY; lsum[q] = 0.f;
+#pragma unroll
+            for (int t = 0; t < kOutTiles; ++t) oacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+
+        // The loads run one block ahead of the arithmetic: the loads of block kb + 64 are issued before the
+        // matrix work on block kb and land in registers (kw: this thread's pieces of the key rows, vw: its
+        // 4 keys x 8 columns of values) while that work runs.  All loads of a block sit in one branch-free
+        // sequence (index clamped, value selected afterwards): loads behind a branch wait one by one.
+        u32x4 kw[NK], vw[4];
+        auto fetch = [&](int kb) {
+            const bool full = kb + kAttKeys <= N;      // uniform: every row of the block exists
+            if constexpr (VEC) {
+                if (full) {
+                    const uint32_t base = (uint32_t)kb * (uint32_t)K;
+#pragma unroll
+                    for (int step = 0; step < NK; ++step)
+                        kw[step] = *reinterpret_cast<const u32x4_unaligned *>(ks + (base + k_off[step]));
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        vw[i] = *reinterpret_cast<const u32x4_unaligned *>(vs + (base + v_off + (uint32_t)(i * K)));
+                } else {
+#pragma unroll
+                    for (int step = 0; step < NK; ++step) {
+                        const int u = step * kAttThreads + tid;
+                        const uint32_t row = (uint32_t)min(kb + u / kPieces, N - 1);
+                        kw[step] = *reinterpret_cast<const u32x4_unaligned *>(ks + (row * (uint32_t)K + k_col[step]));
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t row = (uint32_t)min(kb + 4 * v_kg + i, N - 1);   // threads that do not store load a clamped row
+                        vw[i] = *reinterpret_cast<const u32x4_unaligned *>(vs + (row * (uint32_t)K + v_col));
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int step = 0; step < NK; ++step) {
+                    const int u = step * kAttThreads + tid;
+                    kw[step] = load8_slow(ks + (int64_t)min(kb + u / kPieces, N - 1) * K, 8 * (u % kPieces), K);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    vw[i] = load8_slow(vs + (int64_t)min(kb + 4 * v_kg + i, N - 1) * K, 8 * v_piece, K);
+            }
+            // zeros past the head dimension and past the last key (values: their probabilities are zeros
+            // too, but 0 * stale bits could be NaN)
+            if (!full || K != KP) {
+#pragma unroll
+                for (int step = 0; step < NK; ++step) {
+                    const int u = step * kAttThreads + tid;
+                    kw[step] = (kb + u / kPieces < N && 8 * (u % kPieces) < K) ? kw[step] : zero4;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) vw[i] = (kb + 4 * v_kg + i < N && 8 * v_piece < K) ? vw[i] : zero4;
+            }
+        };
+        if (N > 0) fetch(0);
+
+        for (int kb = 0; kb < N; kb += kAttKeys) {
+            __syncthreads();                           // the previous block (or round) is consumed
+            // ---- keys: sK[key][k], one 16-byte piece per thread and step, pieces of a row on neighbouring lanes
+#pragma unroll
+            for (int step = 0; step < NK; ++step) {
+                const int u = step * kAttThreads + tid;
+                *reinterpret_cast<u32x4 *>(sK + (u / kPieces) * kPitchK + (u % kPieces) * 16) = kw[step];
+            }
+            // ---- values, transposed: 8 runs of 4 keys, one per column of the thread's piece
+            if (v_thread) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {          // word w of the four rows = columns 2w and 2w + 1
+                    const uint32_t lo01 = __builtin_amdgcn_perm(vw[1][w], vw[0][w], 0x05040100u);
+                    const uint32_t lo23 = __builtin_amdgcn_perm(vw[3][w], vw[2][w], 0x05040100u);
+                    const uint32_t hi01 = __builtin_amdgcn_perm(vw[1][w], vw[0][w], 0x07060302u);
+                    const uint32_t hi23 = __builtin_amdgcn_perm(vw[3][w], vw[2][w], 0x07060302u);
+                    unsigned char *dst = sV + (8 * v_piece + 2 * w) * kAttPitchV + v_kg * 8;
+                    *reinterpret_cast<u32x2 *>(dst) = u32x2{lo01, lo23};
+                    *reinterpret_cast<u32x2 *>(dst + kAttPitchV) = u32x2{hi01, hi23};
+                }
+            }
+            __syncthreads();
+            if (kb + kAttKeys < N) fetch(kb + kAttKeys);
+            if (nq == 0) continue;
+
+            // ---- scores of 64 keys x 16 queries per strip; a key operand read serves every strip
+            f32x4 sacc[QT][4];
+#pragma unroll
+            for (int q = 0; q < QT; ++q)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) sacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NK; ++s) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const u32x4 kf = *reinterpret_cast<const u32x4 *>(sK + (16 * t + j) * kPitchK + (4 * s + rg) * 16);
+#pragma unroll
+                    for (int q = 0; q < QT; ++q)
+                        if (QT == 1 || q < nq) sacc[q][t] = Elem<DT>::mfma(kf, qf[q][s], sacc[q][t]);
+                }
+                // keep the operand reads of later steps where they are: moved up front they cost registers
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- online softmax; lane holds keys kb + 16 t + 4 rg + e of query j of each strip
+            const int left = N - kb;                   // keys of this block that exist
+            u32x4 pf[QT][2];
+#pragma unroll
+            for (int q = 0; q < QT; ++q) {
+                if (QT > 1 && q >= nq) continue;
+                f32x4(&sc)[4] = sacc[q];
+                float bm = -INFINITY;
+                if (left < kAttKeys) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) sc[t][e] = 16 * t + 4 * rg + e < left ? sc[t][e] : -INFINITY;
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) bm = fmaxf(bm, sc[t][e]);
+                bm = quad_column_max(bm);
+                const float m_new = fmaxf(m[q], bm);
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = m[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[q] - m_use) * c);
+                m[q] = m_new;
+                const float bias = -m_use * c;
+                float psum = 0.f;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float p = __builtin_amdgcn_exp2f(fmaf(sc[t][e], c, bias));
+                        if (left < kAttKeys) p = 16 * t + 4 * rg + e < left ? p : 0.f;   // also when c = 0
+                        sc[t][e] = p;
+                        psum += p;
+                    }
+                lsum[q] = fmaf(lsum[q], alpha, psum);
+                if (__any(alpha != 1.0f)) {          // the running maxima of long rows settle after a few blocks
+#pragma unroll
+                    for (int t = 0; t < kOutTiles; ++t) oacc[q][t] *= alpha;
+                }
+                // probabilities as B operand, 32 keys per step: k = 8 rg + kk is key 32 cc + 4 rg + kk (kk < 4)
+                // or 32 cc + 16 + 4 rg + kk - 4: what the lane holds in sc[2 cc] and sc[2 cc + 1]
+#pragma unroll
+                for (int cc = 0; cc < 2; ++cc)
+                    pf[q][cc] = u32x4{Elem<DT>::pack2(sc[2 * cc][0], sc[2 * cc][1]), Elem<DT>::pack2(sc[2 * cc][2], sc[2 * cc][3]),
+                                      Elem<DT>::pack2(sc[2 * cc + 1][0], sc[2 * cc + 1][1]),
+                                      Elem<DT>::pack2(sc[2 * cc + 1][2], sc[2 * cc + 1][3])};
+            }
+            // ---- O^T += V^T P^T; a value operand read serves every strip
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc) {
+#pragma unroll
+                for (int t = 0; t < kOutTiles; ++t) {
+                    const unsigned char *vrow = sV + (16 * t + j) * kAttPitchV + (32 * cc + 4 * rg) * 2;
+                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vrow);
+                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vrow + 32);
+                    const u32x4 vf = u32x4{lo[0], lo[1], hi[0], hi[1]};
+#pragma unroll
+                    for (int q = 0; q < QT; ++q)
+                        if (QT == 1 || q < nq) oacc[q][t] = Elem<DT>::mfma(vf, pf[q][cc], oacc[q][t]);
+                    if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        // ---- normalise and store: lane (query j, rg) holds columns 16 t + 4 rg + e.  No key at all: zeros.
+#pragma unroll
+        for (int q = 0; q < QT; ++q) {
+            if (q >= nq) continue;
+            const int qr = r0 + kAttRows * q + j;
+            const float l = quad_column_sum(lsum[q]);
+            const float inv = N > 0 ? 1.0f / l : 0.f;
+            if (qr < M) {
+                uint16_t *orow = os + (int64_t)qr * K;
+#pragma unroll
+                for (int t = 0; t < kOutTiles; ++t) {
+                    const int c0 = 16 * t + 4 * rg;
+                    if (c0 + 4 <= K) {
+                        *reinterpret_cast<u32x2_unaligned *>(orow + c0) =
+                            u32x2{Elem<DT>::pack2(oacc[q][t][0] * inv, oacc[q][t][1] * inv),
+                                  Elem<DT>::pack2(oacc[q][t][2] * inv, oacc[q][t][3] * inv)};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (c0 + e < K) orow[c0 + e] = Elem<DT>::from_float(oacc[q][t][e] * inv);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int DT, int NK, int QT>
+__global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 2 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
+    constexpr int KP = 32 * NK;
+    __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 16)];
+    __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
+    if (!header_ok(a)) { report_mismatch(a); return; }
+    const int g = blockIdx.x;
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
+    const SegRec rec = load_rec(pv.recs, g);
+    const int M = rec.M, K = rec.K;
+    if (M < 1 || K < 1) return;
+    // the launch was sized for a smaller head dimension, or element offsets inside the segment pass 32 bits
+    if (K > KP || (int64_t)max(M, rec.N) * K >= (int64_t(1) << 31)) {
+        if (blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+            atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+        return;
+    }
+    if ((K & 7) == 0) attention_body<DT, NK, QT, true>(a, Vbuf, rec, sK, sV);
+    else attention_body<DT, NK, QT, false>(a, Vbuf, rec, sK, sV);
+}
+
+template <int DT, int QT>
+static void launch_nk(int nk, dim3 grid, hipStream_t stream, const RunArgs &args, const void *V) {
+    switch (nk) {
+        case 1: hipLaunchKernelGGL((attention_kernel<DT, 1, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
+        case 2: hipLaunchKernelGGL((attention_kernel<DT, 2, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
+        case 3: hipLaunchKernelGGL((attention_kernel<DT, 3, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
+        default: hipLaunchKernelGGL((attention_kernel<DT, 4, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
+    }
+}
+
+// Strips per wavefront: two where segments are tall (each operand read from LDS then feeds two matrix
+// instructions and a block of keys is staged half as often), one otherwise (more, lighter workgroups).
+
+int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg, const ba_plan_info *info,
+                     hipStream_t stream) {
+    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
+    if (args.H > 65535) return BA_ERR_UNSUPPORTED;     // heads ride on gridDim.y
+    static const int forced = [] { const char *e = getenv("BLOCKEDATTN_ATT_STRIPS"); return e ? atoi(e) : 0; }();
+    int nk = 4, qt = 1;
+    int64_t max_m = 512;
+    if (info) {
+        if (info->max_K > 128) return BA_ERR_UNSUPPORTED;
+        nseg = info->nseg;
+        nk = std::max(1, (info->max_K + 31) / 32);
+        max_m = std::max<int64_t>(info->max_M, 1);
+        if (info->total_rows >= 128 * std::max<int64_t>(nseg, 1)) qt = 2;   // mean segment height >= 128
+    }
+    if (forced == 1 || forced == 2) qt = forced;
+    const int64_t round_rows = kAttRows * qt;
+    const int64_t z = std::max<int64_t>(1, std::min<int64_t>((max_m + round_rows - 1) / round_rows, 64));
+    if (nseg <= 0) return BA_OK;
+    const dim3 grid((unsigned)nseg, (unsigned)args.H, (unsigned)z);
+    if (dtype == BA_F16) { if (qt == 2) launch_nk<0, 2>(nk, grid, stream, args, V); else launch_nk<0, 1>(nk, grid, stream, args, V); }
+    else { if (qt == 2) launch_nk<1, 2>(nk, grid, stream, args, V); else launch_nk<1, 1>(nk, grid, stream, args, V); }
+    return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+}
+
+}  // namespace ba

@@ -58,6 +58,11 @@ int launch_repack(const void *src_plan, int src_which, int swap_dims, int column
                   int dst_which, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc, int64_t Ddst,
                   const ba_plan_info *dst_info, hipStream_t stream);
 
+// Varlen attention O = softmax(scale Q K^T) V without the probabilities in memory (see attention.hip).
+// args.A = Q, args.B = K, args.out = O ([H, Dm1]); V has K's layout.
+int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg, const ba_plan_info *info,
+                     hipStream_t stream);
+
 // Number of compute units of the current device (cached per device).
 int device_cu_count();
 

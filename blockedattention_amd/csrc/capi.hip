@@ -171,4 +171,17 @@ __attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_
     return launch_strips(dtype, 1, args, nseg, info, (hipStream_t)stream);
 }
 
+__attribute__((visibility("default"))) int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg,
+                                                               int dtype, const void *Q, const void *K,
+                                                               const void *V, void *out, int64_t H, int64_t Dm1,
+                                                               int64_t Dm2, int64_t Dout, float scale,
+                                                               ba_stream_t stream) {
+    if (!plan || nseg < 0 || nseg > (int64_t(1) << 30) || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
+    if (H == 0 || Dm1 == 0 || nseg == 0) return BA_OK;
+    if (!out || !Q || (Dm2 > 0 && (!K || !V))) return BA_ERR_INVALID_ARG;
+    RunArgs args{plan, Q, K, out, H, Dm1, Dm2, Dout, scale, 0, 0, 0, (int)nseg};
+    return launch_attention(dtype, args, V, nseg, info, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -446,6 +446,32 @@ Tensor sparseBlockedGEMMSoftmax_op(const Tensor &mat1, const Tensor &mat2, const
     return out;
 }
 
+// softmax(scale * Q_g K_g^T) V_g in one pass: forward only, the probabilities are never written.
+// Q is the M x K operand of the segments, K and V are both N x K; the result has Q's shape.
+Tensor sparseBlockedAttention_op(const Tensor &q, const Tensor &k, const Tensor &v, const OptTensor &mat1Accum,
+                                 const OptTensor &mat2Accum, const OptTensor &outAccum, const OptTensor &MList,
+                                 const OptTensor &NList, const OptTensor &KList, double scale) {
+    check_data(q, "q"); check_data(k, "k"); check_data(v, "v");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+    TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type(),
+                "q, k and v must have the same dtype");
+    TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16,
+                "the one-pass attention takes fp16 or bf16 operands");
+    TORCH_CHECK(q.device() == k.device() && q.device() == v.device(), "q, k and v must be on the same device");
+    Schedule s = schedule_gemm(q, mat1Accum, mat2Accum, outAccum, MList, NList, KList);
+    TORCH_CHECK(q.size(-1) == s.info.Dm1 && k.size(-1) == s.info.Dm2 && v.size(-1) == s.info.Dm2,
+                "operand sizes do not match the segments: need ", s.info.Dm1, " (q) and ", s.info.Dm2, " (k, v)");
+    TORCH_CHECK(s.info.max_K <= 128, "the one-pass attention takes head dimensions up to 128, got ", s.info.max_K);
+    const int64_t H = leading(q);
+    TORCH_CHECK(leading(k) == H && leading(v) == H, "q, k and v disagree on the number of heads");
+    Tensor out = at::empty({H, s.info.Dm1}, q.options());
+    check_status(ba_varlen_attention(s.plan.data_ptr(), &s.info, s.info.nseg, dtype_code(q, "attention"), q.data_ptr(),
+                                     k.data_ptr(), v.data_ptr(), out.data_ptr(), H, s.info.Dm1, s.info.Dm2,
+                                     s.info.Dout, (float)scale, current_stream(q)),
+                 "ba_varlen_attention");
+    return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -453,6 +479,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sparseBlockedSoftmax", &sparseBlockedSoftmax_op, "sparseBlockedSoftmax forward");
     m.def("sparseBlockedSoftmaxScaled", &sparseBlockedSoftmaxScaled_op, "sparseBlockedSoftmax with a fused scale");
     m.def("sparseBlockedGEMMSoftmax", &sparseBlockedGEMMSoftmax_op, "fused sparseBlockedGEMM + softmax forward");
+    m.def("sparseBlockedAttention", &sparseBlockedAttention_op, "softmax(scale q k^T) v per segment, one pass");
     m.def("set_schedule_cache", &set_schedule_cache, "number of schedules kept for repeated metadata (0 = off)");
     m.def("schedule_cache_stats", &schedule_cache_stats, "[hits, misses, entries, capacity]");
 }

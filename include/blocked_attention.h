@@ -190,6 +190,26 @@ int ba_repack_operand(const void *src_plan, int src_which, int swap_dims, int co
                       int dst_which, const ba_plan_info *dst_info, int64_t nseg, int dtype, const void *src, void *dst,
                       int64_t H, int64_t Dsrc, int64_t Ddst, ba_stream_t stream);
 
+/*
+ * Varlen attention in one pass: out_g = softmax(scale * Q_g K_g^T) V_g per
+ * segment and head, the M x N probabilities never written to memory.  It
+ * stands in for the chain a caller of the reference runs for attention
+ * (README.md:3): sparseBlockedGEMMLaunch, sparseBlockedSoftmaxLaunch and
+ * sparseBlockedGEMMLaunch again with transpose2 on the values
+ * (csrc/sparseBlockedAttention.h:18-20); the reference has no fused form.
+ * Takes a plan from ba_plan_gemm over (M, N, K): Q_g is the M x K operand
+ * (accum1 offsets, Dm1 per head), K_g and V_g are both N x K (accum2 offsets,
+ * Dm2 per head), out_g is M x K at accum1 offsets of an [H, Dm1] buffer.  Dout
+ * is the plan's third total (checked, nothing of that size is touched).
+ * Every K_g <= 128 (larger: BA_ERR_UNSUPPORTED with info, a run error in the
+ * plan without); any alignment.  N_g = 0 gives zeros.  The probabilities are
+ * rounded to dtype before the second product; sums are fp32.
+ * dtype: BA_F16 or BA_BF16.
+ */
+int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg, int dtype, const void *Q, const void *K,
+                        const void *V, void *out, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout, float scale,
+                        ba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -9,6 +9,11 @@ Two independent statements of the same results live here:
 * ``per_segment_torch`` -- one ``torch.matmul`` + ``torch.softmax`` per head and
   segment in fp32, the CPU path the benchmark times beside the GPU.
 
+``attention`` / ``per_segment_torch_attention`` state the one-pass attention
+(probabilities times values) the same two ways; tests/test_oracle_values.py pins
+them with closed forms (uniform scores give column means, one-hot values return
+the probabilities, a dominant key returns its value row) and a brute-force loop.
+
 Both follow the semantics of the reference at
 csrc/sparseBlockedAttention.cpp:11-50, 81-101, csrc/cuda/spBlkGEMM.cu:133-150,
 292-329, 363-400, 985-1008 and csrc/cuda/spBlkSoftmax.cu:95-136, 375-398.
@@ -168,6 +173,15 @@ def gemm_softmax(A, Bm, M, N, K, scale=1.0, return_scores=False):
     return (probs, scores) if return_scores else probs
 
 
+def attention(Q, Km, V, M, N, K, scale=1.0):
+    """O_g = softmax(scale * Q_g K_g^T) V_g in the C loops: the fused pair above, then the varlen GEMM
+    again with the probabilities as the M x N operand (reduction over N) and V_g (N x K, i.e. stored
+    "reduction x columns") as the transposed second operand -- the chain a caller of the reference runs
+    (README.md:3; csrc/cuda/spBlkGEMM.cu:363-400 for transpose2).  fp32 [H, sum(M*K)]."""
+    probs = gemm_softmax(Q, Km, M, N, K, scale)
+    return varlen_gemm(probs, V, M, K, N, transpose2=True)
+
+
 # ---------------------------------------------- per-segment torch (CPU baseline)
 def per_segment_torch(A, Bm, M, N, K, scale=1.0, want="probs"):
     """One fp32 torch.matmul (+ torch.softmax) per head and segment on host tensors.
@@ -206,4 +220,22 @@ def per_segment_torch_softmax(src, rows, cols, scale=1.0):
     for r, c in zip([int(v) for v in rows], [int(v) for v in cols]):
         out[:, o:o + r * c] = torch.softmax(src[:, o:o + r * c].reshape(H, r, c) * scale, -1).reshape(H, r * c)
         o += r * c
+    return out
+
+
+def per_segment_torch_attention(Q, Km, V, M, N, K, scale=1.0):
+    """softmax(scale * Q_g K_g^T) V_g with one fp32 torch.matmul / softmax / matmul per segment."""
+    import torch
+    Q = Q.float(); Km = Km.float(); V = V.float()
+    H = Q.shape[0]
+    out = torch.zeros_like(Q)
+    o1 = o2 = 0
+    for m, n, k in zip([int(v) for v in M], [int(v) for v in N], [int(v) for v in K]):
+        q = Q[:, o1:o1 + m * k].reshape(H, m, k)
+        kk = Km[:, o2:o2 + n * k].reshape(H, n, k)
+        vv = V[:, o2:o2 + n * k].reshape(H, n, k)
+        if n > 0:
+            p = torch.softmax(torch.matmul(q, kk.transpose(1, 2)) * scale, dim=-1)
+            out[:, o1:o1 + m * k] = torch.matmul(p, vv).reshape(H, m * k)
+        o1 += m * k; o2 += n * k
     return out

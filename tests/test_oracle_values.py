@@ -130,3 +130,75 @@ def test_c_oracle_and_per_segment_torch_agree(cfg):
     np.testing.assert_allclose(pr_c, pr_t.numpy(), rtol=1e-4, atol=1e-6)
     ref = oracle.per_segment_torch_softmax(sc_t, w.M, w.N, w.scale)
     np.testing.assert_allclose(ref.numpy(), pr_t.numpy(), rtol=1e-6, atol=1e-8)
+
+
+# ------------------------------------------------------------------ attention (probabilities times values)
+def _attention_inputs(seed, M, N, K, H=2):
+    rng = np.random.default_rng(seed)
+    M, N, K = np.asarray(M), np.asarray(N), np.asarray(K)
+    Q = rng.standard_normal((H, int((M * K).sum()))).astype(np.float32)
+    Km = rng.standard_normal((H, int((N * K).sum()))).astype(np.float32)
+    V = rng.standard_normal((H, int((N * K).sum()))).astype(np.float32)
+    return Q, Km, V, M, N, K
+
+
+def test_attention_brute_force_loops():
+    # plain Python in float64, index by index: a transposed operand or a wrong offset changes it
+    Q, Km, V, M, N, K = _attention_inputs(3, [3, 1, 4], [5, 2, 3], [2, 4, 3])
+    scale = 0.7
+    got = oracle.attention(Q, Km, V, M, N, K, scale)
+    expect = np.zeros_like(got, dtype=np.float64)
+    for h in range(Q.shape[0]):
+        o1 = o2 = 0
+        for m, n, k in zip(M, N, K):
+            for r in range(m):
+                s = [scale * sum(float(Q[h, o1 + r * k + t]) * float(Km[h, o2 + c * k + t]) for t in range(k)) for c in range(n)]
+                e = [np.exp(x - max(s)) for x in s]
+                for d in range(k):
+                    expect[h, o1 + r * k + d] = sum(e[c] * float(V[h, o2 + c * k + d]) for c in range(n)) / sum(e)
+            o1 += m * k; o2 += n * k
+    assert np.allclose(got, expect, rtol=1e-5, atol=1e-6)
+
+
+def test_attention_uniform_scores_give_column_means():
+    Q, Km, V, M, N, K = _attention_inputs(4, [4, 2], [6, 9], [8, 3])
+    got = oracle.attention(np.zeros_like(Q), Km, V, M, N, K, 1.0)
+    o1 = o2 = 0
+    for m, n, k in zip(M, N, K):
+        mean = V[:, o2:o2 + n * k].reshape(-1, n, k).mean(axis=1)
+        assert np.allclose(got[:, o1:o1 + m * k].reshape(-1, m, k), mean[:, None, :], atol=1e-6)
+        o1 += m * k; o2 += n * k
+
+
+def test_attention_one_hot_values_return_the_probabilities():
+    # V_g[n][d] = (n == d): O_g = the first K columns of P_g (N <= K pads with zeros)
+    Q, Km, V, M, N, K = _attention_inputs(5, [5, 3], [4, 7], [6, 7])
+    V = np.zeros_like(V)
+    o2 = 0
+    for n, k in zip(N, K):
+        V[:, o2:o2 + n * k] = np.eye(n, k, dtype=np.float32).ravel()
+        o2 += n * k
+    got = oracle.attention(Q, Km, V, M, N, K, 0.5)
+    probs = oracle.gemm_softmax(Q, Km, M, N, K, 0.5)
+    o1 = oo = 0
+    for m, n, k in zip(M, N, K):
+        P = probs[:, oo:oo + m * n].reshape(-1, m, n)
+        want = np.zeros((Q.shape[0], m, k), np.float32)
+        want[:, :, :min(n, k)] = P[:, :, :min(n, k)]
+        assert np.allclose(got[:, o1:o1 + m * k].reshape(-1, m, k), want, atol=1e-6)
+        o1 += m * k; oo += m * n
+
+
+def test_attention_dominant_key_returns_its_value_row():
+    Q, Km, V, M, N, K = _attention_inputs(6, [3], [5], [4], H=1)
+    Km[:] = 0.0
+    Km[0, 2 * 4:3 * 4] = 100.0 * np.sign(Q[0, :4])          # key 2 dominates query 0
+    got = oracle.attention(Q, Km, V, M, N, K, 1.0)
+    assert np.allclose(got[0, :4], V[0, 2 * 4:3 * 4], atol=1e-4)
+
+
+def test_attention_two_statements_agree():
+    Q, Km, V, M, N, K = _attention_inputs(7, [9, 0, 17, 5], [12, 4, 0, 33], [8, 16, 5, 24], H=3)
+    a = oracle.attention(Q, Km, V, M, N, K, 0.3)
+    b = oracle.per_segment_torch_attention(torch.from_numpy(Q), torch.from_numpy(Km), torch.from_numpy(V), M, N, K, 0.3)
+    assert np.allclose(a, b.numpy(), rtol=1e-5, atol=1e-6)
