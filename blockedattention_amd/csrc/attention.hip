@@ -59,8 +59,8 @@ __device__ __forceinline__ u32x4 load8_slow(const uint16_t *row, int k0, int K) 
 // rows come as 16-byte loads; otherwise element by element.  The two are separate instances of the whole
 // body so that the slow loads do not sit inside the fast path's loops.
 template <int DT, int NK, int QT, bool VEC>
-__device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbuf, const SegRec &rec, unsigned char *sK,
-                                               unsigned char *sV) {
+__device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbuf, const SegRec &rec, int64_t h, int zblock,
+                                               unsigned char *sK, unsigned char *sV) {
     constexpr int KP = 32 * NK;                       // padded head dimension
     constexpr int kPitchK = KP * 2 + 16;              // bytes per LDS row of keys (16-byte skew: 16 lanes of
                                                       // a 16-byte read cover all banks once)
@@ -71,7 +71,6 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     const int wave = uniform(tid >> 6);
     const int lane = lane_id();
     const int j = lane & 15, rg = lane >> 4;
-    const int64_t h = blockIdx.y;
     const uint16_t *qs = reinterpret_cast<const uint16_t *>(a.A) + h * a.Dm1 + rec.off1;
     const uint16_t *ks = reinterpret_cast<const uint16_t *>(a.B) + h * a.Dm2 + rec.off2;
     const uint16_t *vs = reinterpret_cast<const uint16_t *>(Vbuf) + h * a.Dm2 + rec.off2;
@@ -101,7 +100,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     const uint32_t v_off = (uint32_t)(4 * v_kg) * (uint32_t)K + v_col;
 
     constexpr int kRoundRows = kAttRows * QT;           // queries per workgroup round
-    for (int round = blockIdx.z; round * kRoundRows < M; round += gridDim.z) {
+    for (int round = zblock; round * kRoundRows < M; round += a.tile_zdim) {
         // strip q of the wavefront: rows round * kRoundRows + 64 q + 16 wave ..; the live ones come first
         const int r0 = round * kRoundRows + wave * 16;
         const int nq = uniform(r0 >= M ? 0 : min(QT, (M - r0 + kAttRows - 1) / kAttRows));   // 0: the wavefront only stages
@@ -325,23 +324,37 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 2 ? 4 : 3) void at
     __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 16)];
     __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
     if (!header_ok(a)) { report_mismatch(a); return; }
-    const int g = blockIdx.x;
+    // Workgroup -> (segment, head, row block).  Consecutive workgroup ids go to the eight dies of the chip in
+    // turn, and each die has its own L2: id = die + 8 k.  All row blocks of one (segment, head) pair read the
+    // same keys and values, so they get consecutive k on ONE die (pair = die + 8 (k / Z), row block k % Z) and
+    // run at about the same time; with the head as the fast index of a pair, every die gets its share of
+    // every segment.
+    // (Short segments, where most pairs have fewer row blocks than Z and nothing to share: row block as the
+    // slow index instead, ride_z = 0, so that the workgroups that find no rows come last.)
+    const unsigned id = blockIdx.x, die = id & 7u, kk = id >> 3;
+    const unsigned Z = (unsigned)a.tile_zdim, pairs8 = (unsigned)a.tile_groups;
+    const int64_t pair = (int64_t)die + 8 * (int64_t)(a.ride_z ? kk / Z : kk % pairs8);
+    const int zblock = (int)(a.ride_z ? kk % Z : kk / pairs8);
+    if (pair >= (int64_t)a.nseg * a.H) return;
+    const int g = (int)(pair / a.H);
+    const int64_t h = pair % a.H;
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     const SegRec rec = load_rec(pv.recs, g);
     const int M = rec.M, K = rec.K;
     if (M < 1 || K < 1) return;
     // the launch was sized for a smaller head dimension, or element offsets inside the segment pass 32 bits
     if (K > KP || (int64_t)max(M, rec.N) * K >= (int64_t(1) << 31)) {
-        if (blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+        if (h == 0 && zblock == 0 && threadIdx.x == 0)
             atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
     }
-    if ((K & 7) == 0) attention_body<DT, NK, QT, true>(a, Vbuf, rec, sK, sV);
-    else attention_body<DT, NK, QT, false>(a, Vbuf, rec, sK, sV);
+    if ((K & 7) == 0) attention_body<DT, NK, QT, true>(a, Vbuf, rec, h, zblock, sK, sV);
+    else attention_body<DT, NK, QT, false>(a, Vbuf, rec, h, zblock, sK, sV);
 }
 
 template <int DT, int QT>
 static void launch_nk(int nk, dim3 grid, hipStream_t stream, const RunArgs &args, const void *V) {
+    // args.tile_zdim = row blocks per (segment, head) pair, tile_groups = pairs per die, ride_z = row block fastest
     switch (nk) {
         case 1: hipLaunchKernelGGL((attention_kernel<DT, 1, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
         case 2: hipLaunchKernelGGL((attention_kernel<DT, 2, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
@@ -356,7 +369,6 @@ static void launch_nk(int nk, dim3 grid, hipStream_t stream, const RunArgs &args
 int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg, const ba_plan_info *info,
                      hipStream_t stream) {
     if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
-    if (args.H > 65535) return BA_ERR_UNSUPPORTED;     // heads ride on gridDim.y
     static const int forced = [] { const char *e = getenv("BLOCKEDATTN_ATT_STRIPS"); return e ? atoi(e) : 0; }();
     int nk = 4, qt = 1;
     int64_t max_m = 512;
@@ -368,12 +380,22 @@ int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg
         if (info->total_rows >= 128 * std::max<int64_t>(nseg, 1)) qt = 2;   // mean segment height >= 128
     }
     if (forced == 1 || forced == 2) qt = forced;
+    // Row blocks per pair: enough for the tallest segment, but no more than four times what the mean segment
+    // needs (a workgroup takes every Z-th block of its pair; blocks that do not exist cost a launch each).
     const int64_t round_rows = kAttRows * qt;
-    const int64_t z = std::max<int64_t>(1, std::min<int64_t>((max_m + round_rows - 1) / round_rows, 64));
+    int64_t z = std::min<int64_t>((max_m + round_rows - 1) / round_rows, 64);
+    if (info) z = std::min<int64_t>(z, (4 * info->total_rows / std::max<int64_t>(nseg, 1) + round_rows - 1) / round_rows);
+    z = std::max<int64_t>(z, 1);
     if (nseg <= 0) return BA_OK;
-    const dim3 grid((unsigned)nseg, (unsigned)args.H, (unsigned)z);
-    if (dtype == BA_F16) { if (qt == 2) launch_nk<0, 2>(nk, grid, stream, args, V); else launch_nk<0, 1>(nk, grid, stream, args, V); }
-    else { if (qt == 2) launch_nk<1, 2>(nk, grid, stream, args, V); else launch_nk<1, 1>(nk, grid, stream, args, V); }
+    const int64_t pairs8 = (nseg * args.H + 7) / 8;    // pairs per die, rounded up
+    if (pairs8 * z * 8 > 0x7fffffff || pairs8 > 0x7fffffff) return BA_ERR_UNSUPPORTED;
+    RunArgs run = args;
+    run.tile_zdim = (int)z;
+    run.tile_groups = (int)pairs8;
+    run.ride_z = (info && info->total_rows >= 512 * nseg) ? 1 : 0;   // tall segments: row blocks of a pair side by side
+    const dim3 grid((unsigned)(pairs8 * z * 8));
+    if (dtype == BA_F16) { if (qt == 2) launch_nk<0, 2>(nk, grid, stream, run, V); else launch_nk<0, 1>(nk, grid, stream, run, V); }
+    else { if (qt == 2) launch_nk<1, 2>(nk, grid, stream, run, V); else launch_nk<1, 1>(nk, grid, stream, run, V); }
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
