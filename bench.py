@@ -87,6 +87,13 @@ class Case:
         self._a_fused = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.out), code,
                          *dims, f32(w.scale), st)
         self.scores = self.torch.empty_like(self.out)
+        # one-pass attention on the same segments: values shaped like the keys, output shaped like the queries
+        g = self.torch.Generator(device="cpu").manual_seed(1)
+        self.V_host = self.torch.randn(self.B_host.shape, generator=g).to(w.dtype)
+        self.V = self.V_host.to(self.dev)
+        self.att = self.torch.empty_like(self.A)
+        self._a_att = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.V),
+                       c._ptr(self.att), *dims, f32(w.scale), st)
         self._a_gemm = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.scores),
                         *dims, i32(0), i32(0), st)
         self._a_soft = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.scores), c._ptr(self.out), i64(w.heads),
@@ -94,7 +101,8 @@ class Case:
         for st_code, what in ((lib.ba_plan_gemm(*self._a_sched), "ba_plan_gemm"),
                               (lib.ba_gemm_softmax(*self._a_fused), "ba_gemm_softmax"),
                               (lib.ba_varlen_gemm(*self._a_gemm), "ba_varlen_gemm"),
-                              (lib.ba_blocked_softmax(*self._a_soft), "ba_blocked_softmax")):
+                              (lib.ba_blocked_softmax(*self._a_soft), "ba_blocked_softmax"),
+                              (lib.ba_varlen_attention(*self._a_att), "ba_varlen_attention")):
             c.check(st_code, what)
 
     def schedule(self):
@@ -108,6 +116,9 @@ class Case:
 
     def softmax(self):
         self._lib.ba_blocked_softmax(*self._a_soft)
+
+    def attention(self):
+        self._lib.ba_varlen_attention(*self._a_att)
 
     def step(self):
         self._lib.ba_plan_gemm(*self._a_sched)
@@ -147,6 +158,7 @@ class Case:
         import numpy as np
         torch, w = self.torch, self.w
         self.step()
+        self.attention()
         torch.cuda.synchronize()
         a1 = self.acc[0].cpu().numpy(); a2 = self.acc[1].cpu().numpy(); ao = self.acc[2].cpu().numpy()
         rng = np.random.default_rng(1)
@@ -163,6 +175,16 @@ class Case:
             if not bool((err <= tol).all()):
                 raise SystemExit(f"parity gate failed on config {self.cfg}, segment {g}, head {h}: {float(err.max())}")
             worst = max(worst, float(err.max()))
+            # one-pass attention on the same segment: fp32 reference, bound from the two 16-bit roundings
+            # (probabilities before the second product, result at the store)
+            v = self.V_host[h, a2[g]:a2[g + 1]].float().reshape(n, k)
+            o = self.att[h, a1[g]:a1[g + 1]].float().cpu().reshape(m, k)
+            u = 2.0 ** -9 if w.dtype == torch.bfloat16 else 2.0 ** -11
+            oref = ref @ v
+            bound = 2 * u * (ref @ v.abs() + oref.abs()) + 1e-3 * float(oref.pow(2).mean().sqrt())
+            if not bool(((o - oref).abs() <= bound).all()):
+                raise SystemExit(f"attention parity gate failed on config {self.cfg}, segment {g}, head {h}: "
+                                 f"{float((o - oref).abs().max())}")
         return worst
 
     def gpu_figures(self, steps, warmup, with_unfused=True):
@@ -178,6 +200,13 @@ class Case:
             "hbm_frac": round(w.pair_bytes() / k_us * 1e-3 / HBM_PEAK_GBS, 4),
             "mfma_frac": round(w.flops / k_us * 1e-6 / MFMA_PEAK_TFLOPS, 4),
         }
+        # one-pass attention: both products counted, queries + keys + values read, outputs written
+        a_us = self.event_us(self.attention, steps, warmup)
+        a_bytes = 2 * w.heads * (2 * w.Dm1 + 2 * w.Dm2)
+        fig["attention"] = {"kernel_us": round(a_us, 3), "bytes": a_bytes, "flops": 2 * w.flops,
+                            "GBps": round(a_bytes / a_us * 1e-3, 1), "TFLOPs": round(2 * w.flops / a_us * 1e-6, 2),
+                            "mfma_frac": round(2 * w.flops / a_us * 1e-6 / MFMA_PEAK_TFLOPS, 4),
+                            "hbm_frac": round(a_bytes / a_us * 1e-3 / HBM_PEAK_GBS, 4)}
         if with_unfused:
             fig["gemm_only_us"] = round(self.event_us(self.gemm, steps, warmup), 3)
             fig["softmax_only_us"] = round(self.event_us(self.softmax, steps, warmup), 3)

@@ -95,10 +95,17 @@ def test_launch_without_the_host_summary(dev):
     run(dev, M, N, K, 2, torch.float16, 0.125, summary=False)
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
 def test_benchmark_configurations(dev, cfg):
+    # configuration 5 (segments of 1024 .. 4096 rows) at full segment sizes on one head
     w = workloads.make(cfg)
-    run(dev, w.M, w.N, w.K, min(w.heads, 2), w.dtype, w.scale)
+    run(dev, w.M, w.N, w.K, min(w.heads, 2) if cfg < 5 else 1, w.dtype, w.scale, sigma=w.sigma)
+
+
+def test_tall_segments_row_blocks_side_by_side(dev):
+    # mean height >= 512: two strips per wavefront and the row blocks of a (segment, head) pair on one die
+    run(dev, [600, 1000, 513], [300, 700, 64], [64, 64, 64], 3, torch.float16, 0.125)
+    run(dev, [700, 520], [130, 900], [128, 40], 2, torch.bfloat16, 0.1, seed=4)
 
 
 def test_matches_the_three_call_chain(dev):
