@@ -23,6 +23,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "ba_device.hpp"
 #include "ba_gemm_common.hpp"
@@ -209,87 +210,89 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
             __syncthreads();
             if (kb + kAttKeys < N) fetch(kb + kAttKeys);
             if (nq == 0) continue;
-
-            // ---- scores of 64 keys x 16 queries per strip; a key operand read serves every strip
-            f32x4 sacc[QT][4];
-#pragma unroll
-            for (int q = 0; q < QT; ++q)
-#pragma unroll
-                for (int t = 0; t < 4; ++t) sacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < NK; ++s) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const u32x4 kf = *reinterpret_cast<const u32x4 *>(sK + (16 * t + j) * kPitchK + (4 * s + rg) * 16);
-#pragma unroll
-                    for (int q = 0; q < QT; ++q)
-                        if (QT == 1 || q < nq) sacc[q][t] = Elem<DT>::mfma(kf, qf[q][s], sacc[q][t]);
-                }
-                // keep the operand reads of later steps where they are: moved up front they cost registers
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // ---- online softmax; lane holds keys kb + 16 t + 4 rg + e of query j of each strip
-            const int left = N - kb;                   // keys of this block that exist
-            u32x4 pf[QT][2];
-#pragma unroll
-            for (int q = 0; q < QT; ++q) {
-                if (QT > 1 && q >= nq) continue;
-                f32x4(&sc)[4] = sacc[q];
-                float bm = -INFINITY;
-                if (left < kAttKeys) {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) sc[t][e] = 16 * t + 4 * rg + e < left ? sc[t][e] : -INFINITY;
-                }
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) bm = fmaxf(bm, sc[t][e]);
-                bm = quad_column_max(bm);
-                const float m_new = fmaxf(m[q], bm);
-                const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                const float alpha = m[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[q] - m_use) * c);
-                m[q] = m_new;
-                const float bias = -m_use * c;
-                float psum = 0.f;
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        float p = __builtin_amdgcn_exp2f(fmaf(sc[t][e], c, bias));
-                        if (left < kAttKeys) p = 16 * t + 4 * rg + e < left ? p : 0.f;   // also when c = 0
-                        sc[t][e] = p;
-                        psum += p;
+            // The arithmetic on one block for NQ live strips, as straight-line code: a branch around every
+            // matrix instruction of a strip that may be missing would keep the scheduler from interleaving them.
+            auto block_math = [&](auto nq_tag) {
+                constexpr int NQ = decltype(nq_tag)::value;
+                // ---- scores of 64 keys x 16 queries per strip; a key operand read serves every strip
+                f32x4 sacc[NQ][4];
+    #pragma unroll
+                for (int q = 0; q < NQ; ++q)
+    #pragma unroll
+                    for (int t = 0; t < 4; ++t) sacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                for (int s = 0; s < NK; ++s) {
+    #pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const u32x4 kf = *reinterpret_cast<const u32x4 *>(sK + (16 * t + j) * kPitchK + (4 * s + rg) * 16);
+    #pragma unroll
+                        for (int q = 0; q < NQ; ++q)
+                            sacc[q][t] = Elem<DT>::mfma(kf, qf[q][s], sacc[q][t]);
                     }
-                lsum[q] = fmaf(lsum[q], alpha, psum);
-                if (__any(alpha != 1.0f)) {          // the running maxima of long rows settle after a few blocks
-#pragma unroll
-                    for (int t = 0; t < kOutTiles; ++t) oacc[q][t] *= alpha;
                 }
-                // probabilities as B operand, 32 keys per step: k = 8 rg + kk is key 32 cc + 4 rg + kk (kk < 4)
-                // or 32 cc + 16 + 4 rg + kk - 4: what the lane holds in sc[2 cc] and sc[2 cc + 1]
-#pragma unroll
-                for (int cc = 0; cc < 2; ++cc)
-                    pf[q][cc] = u32x4{Elem<DT>::pack2(sc[2 * cc][0], sc[2 * cc][1]), Elem<DT>::pack2(sc[2 * cc][2], sc[2 * cc][3]),
-                                      Elem<DT>::pack2(sc[2 * cc + 1][0], sc[2 * cc + 1][1]),
-                                      Elem<DT>::pack2(sc[2 * cc + 1][2], sc[2 * cc + 1][3])};
-            }
-            // ---- O^T += V^T P^T; a value operand read serves every strip
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc) {
-#pragma unroll
-                for (int t = 0; t < kOutTiles; ++t) {
-                    const unsigned char *vrow = sV + (16 * t + j) * kAttPitchV + (32 * cc + 4 * rg) * 2;
-                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vrow);
-                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vrow + 32);
-                    const u32x4 vf = u32x4{lo[0], lo[1], hi[0], hi[1]};
-#pragma unroll
-                    for (int q = 0; q < QT; ++q)
-                        if (QT == 1 || q < nq) oacc[q][t] = Elem<DT>::mfma(vf, pf[q][cc], oacc[q][t]);
-                    if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                // ---- online softmax; lane holds keys kb + 16 t + 4 rg + e of query j of each strip
+                const int left = N - kb;                   // keys of this block that exist
+                u32x4 pf[NQ][2];
+    #pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    f32x4(&sc)[4] = sacc[q];
+                    float bm = -INFINITY;
+                    if (left < kAttKeys) {
+    #pragma unroll
+                        for (int t = 0; t < 4; ++t)
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e) sc[t][e] = 16 * t + 4 * rg + e < left ? sc[t][e] : -INFINITY;
+                    }
+    #pragma unroll
+                    for (int t = 0; t < 4; ++t)
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) bm = fmaxf(bm, sc[t][e]);
+                    bm = quad_column_max(bm);
+                    const float m_new = fmaxf(m[q], bm);
+                    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                    const float alpha = m[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[q] - m_use) * c);
+                    m[q] = m_new;
+                    const float bias = -m_use * c;
+                    float psum = 0.f;
+    #pragma unroll
+                    for (int t = 0; t < 4; ++t)
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float p = __builtin_amdgcn_exp2f(fmaf(sc[t][e], c, bias));
+                            if (left < kAttKeys) p = 16 * t + 4 * rg + e < left ? p : 0.f;   // also when c = 0
+                            sc[t][e] = p;
+                            psum += p;
+                        }
+                    lsum[q] = fmaf(lsum[q], alpha, psum);
+                    if (__any(alpha != 1.0f)) {          // the running maxima of long rows settle after a few blocks
+    #pragma unroll
+                        for (int t = 0; t < kOutTiles; ++t) oacc[q][t] *= alpha;
+                    }
+                    // probabilities as B operand, 32 keys per step: k = 8 rg + kk is key 32 cc + 4 rg + kk (kk < 4)
+                    // or 32 cc + 16 + 4 rg + kk - 4: what the lane holds in sc[2 cc] and sc[2 cc + 1]
+    #pragma unroll
+                    for (int cc = 0; cc < 2; ++cc)
+                        pf[q][cc] = u32x4{Elem<DT>::pack2(sc[2 * cc][0], sc[2 * cc][1]), Elem<DT>::pack2(sc[2 * cc][2], sc[2 * cc][3]),
+                                          Elem<DT>::pack2(sc[2 * cc + 1][0], sc[2 * cc + 1][1]),
+                                          Elem<DT>::pack2(sc[2 * cc + 1][2], sc[2 * cc + 1][3])};
                 }
-            }
+                // ---- O^T += V^T P^T; a value operand read serves every strip
+    #pragma unroll
+                for (int cc = 0; cc < 2; ++cc) {
+    #pragma unroll
+                    for (int t = 0; t < kOutTiles; ++t) {
+                        const unsigned char *vrow = sV + (16 * t + j) * kAttPitchV + (32 * cc + 4 * rg) * 2;
+                        const u32x2 lo = *reinterpret_cast<const u32x2 *>(vrow);
+                        const u32x2 hi = *reinterpret_cast<const u32x2 *>(vrow + 32);
+                        const u32x4 vf = u32x4{lo[0], lo[1], hi[0], hi[1]};
+    #pragma unroll
+                        for (int q = 0; q < NQ; ++q)
+                            oacc[q][t] = Elem<DT>::mfma(vf, pf[q][cc], oacc[q][t]);
+                    }
+                }
+            };
+            if (QT == 1 || nq == 1) block_math(std::integral_constant<int, 1>{});
+            else block_math(std::integral_constant<int, QT>{});
         }
         // ---- normalise and store: lane (query j, rg) holds columns 16 t + 4 rg + e.  No key at all: zeros.
 #pragma unroll
@@ -319,7 +322,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
 }
 
 template <int DT, int NK, int QT>
-__global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 2 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
+__global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
     constexpr int KP = 32 * NK;
     __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 16)];
     __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
