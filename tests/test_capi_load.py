@@ -51,6 +51,10 @@ def test_argument_errors_are_reported_without_a_device():
     assert lib.ba_gemm_softmax(p, None, 1, 2, p, p, p, 2, 1, 8, 8, 1, 1.0, null) == 3                # fp32 operands
     assert lib.ba_gemm_softmax(p, None, 1, 0, p, p, p, 1, 1, 8, 8, 1, 1.0, null) == 3                # f16 in, bf16 out
     assert lib.ba_blocked_softmax(null, None, 1, 0, null, null, 1, 1, 1.0, null) == 1
+    assert lib.ba_varlen_attention(p, None, 1, 2, p, p, p, p, 1, 8, 8, 1, 1.0, null) == 3            # fp32 operands
+    assert lib.ba_varlen_attention(p, None, 1, 0, p, p, null, p, 1, 8, 8, 1, 1.0, null) == 1         # no values
+    assert lib.ba_varlen_attention(null, None, 1, 0, p, p, p, p, 1, 8, 8, 1, 1.0, null) == 1         # no plan
+    assert lib.ba_varlen_attention(p, None, 0, 0, p, p, p, p, 1, 8, 8, 1, 1.0, null) == 0            # no segments
     # empty work is not an error and launches nothing
     assert lib.ba_varlen_gemm(p, None, 1, 0, null, null, null, 0, 0, 0, 0, 0, 0, null) == 0
     assert lib.ba_blocked_softmax(p, None, 1, 0, null, null, 4, 0, 1.0, null) == 0
