@@ -14,8 +14,9 @@
 //   S^T block  = K_blk Q^T   (matrix instructions, A operand = key rows from LDS, B operand = the
 //                wavefront's query rows, held in registers for the whole pass); the lane
 //                (j = lane%16, rg = lane/16) then holds query j's scores for keys 16t + 4rg + e;
-//   online softmax: running row maximum m and row sum l per query (per lane; the four lanes of a
-//                query exchange the block maximum), accumulators rescaled by 2^((m_old - m_new) c);
+//   online softmax: reference value m (a lazily raised row maximum) and row sum l per query (per lane;
+//                the four lanes of a query exchange the block maximum), accumulators rescaled by
+//                2^((m_old - m_new) c) when m is raised;
 //   O^T       += V_blk^T P^T (A operand = transposed value rows from LDS, B operand = the lane's own
 //                probabilities rounded to the 16-bit type: the k index of the instruction runs over
 //                keys in the order the score registers hold them, so P never moves between lanes).
@@ -248,9 +249,15 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     #pragma unroll
                         for (int e = 0; e < 4; ++e) bm = fmaxf(bm, sc[t][e]);
                     bm = quad_column_max(bm);
-                    const float m_new = fmaxf(m[q], bm);
+                    // m is the reference the exponentials are taken against, not necessarily the maximum: it is
+                    // raised (and the sums so far rescaled) only when a block's maximum passes it by more than
+                    // 2^8 in the exponent, so probabilities stay below 256 (fine for both 16-bit types and the
+                    // fp32 sums) and most blocks skip the rescale.  The comparison is false, i.e. raises, for the
+                    // first block (m = -inf).
+                    const bool raise = !((bm - m[q]) * c <= 8.0f);
+                    const float m_new = raise ? bm : m[q];
                     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                    const float alpha = m[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[q] - m_use) * c);
+                    const float alpha = !raise ? 1.0f : m[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[q] - m_use) * c);
                     m[q] = m_new;
                     const float bias = -m_use * c;
                     float psum = 0.f;
@@ -264,7 +271,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
                             psum += p;
                         }
                     lsum[q] = fmaf(lsum[q], alpha, psum);
-                    if (__any(alpha != 1.0f)) {          // the running maxima of long rows settle after a few blocks
+                    if (__any(raise)) {
     #pragma unroll
                         for (int t = 0; t < kOutTiles; ++t) oacc[q][t] *= alpha;
                     }
