@@ -36,6 +36,7 @@ constexpr int kAttThreads = 256;
 constexpr int kAttWaves = kAttThreads / 64;
 constexpr int kAttKeys = 64;                          // keys per block
 constexpr int kAttRows = 16 * kAttWaves;              // queries per workgroup round
+static_assert(kAttRows == kAttBlockRows, "the plan's row-block prefixes count blocks of kAttRows and 2 kAttRows");
 constexpr int kAttPitchV = kAttKeys * 2 + 8;          // bytes per LDS row of transposed values.  An LDS access
 // serves 16 lanes x 8 bytes at a time; the 8-byte skew puts the sixteen rows 16 t + j that an operand read
 // touches in sixteen different 8-byte bank groups, and a staging write covers one row's 128 bytes.
@@ -102,7 +103,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     const uint32_t v_off = (uint32_t)(4 * v_kg) * (uint32_t)K + v_col;
 
     constexpr int kRoundRows = kAttRows * QT;           // queries per workgroup round
-    for (int round = zblock; round * kRoundRows < M; round += a.tile_zdim) {
+    for (int round = zblock; (int64_t)round * kRoundRows < M; round += a.ride_slots ? (1 << 24) : a.tile_zdim) {
         // strip q of the wavefront: rows round * kRoundRows + 64 q + 16 wave ..; the live ones come first
         const int r0 = round * kRoundRows + wave * 16;
         const int nq = uniform(r0 >= M ? 0 : min(QT, (M - r0 + kAttRows - 1) / kAttRows));   // 0: the wavefront only stages
@@ -341,13 +342,31 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void at
     // every segment.
     // (Short segments, where most pairs have fewer row blocks than Z and nothing to share: row block as the
     // slow index instead, ride_z = 0, so that the workgroups that find no rows come last.)
+    // With the row-block prefix (ride_slots = 1, launches that know the batch's totals): the existing
+    // (head, segment, row block) items, head-major, are cut into eight contiguous shares, one per die, so the
+    // row blocks of a pair still sit side by side on one die and no workgroup is launched for a row block that
+    // does not exist, except past the end of a share (the grid is sized from an upper bound of the item count).
     const unsigned id = blockIdx.x, die = id & 7u, kk = id >> 3;
-    const unsigned Z = (unsigned)a.tile_zdim, pairs8 = (unsigned)a.tile_groups;
-    const int64_t pair = (int64_t)die + 8 * (int64_t)(a.ride_z ? kk / Z : kk % pairs8);
-    const int zblock = (int)(a.ride_z ? kk % Z : kk / pairs8);
-    if (pair >= (int64_t)a.nseg * a.H) return;
-    const int g = (int)(pair / a.H);
-    const int64_t h = pair % a.H;
+    int g, zblock;
+    int64_t h;
+    if (a.ride_slots) {
+        const int32_t *pfx = plan_rowblocks(a.plan, a.nseg, QT - 1);
+        const int64_t per_head = ((ConstI32)(uintptr_t)pfx)[a.nseg];
+        const int64_t items = per_head * a.H, share = (items + 7) >> 3;
+        const int64_t u = (int64_t)die * share + kk;
+        if (kk >= share || u >= items) return;
+        h = u / per_head;
+        const int item = (int)(u % per_head);
+        g = prefix_search(pfx, a.nseg, item);
+        zblock = item - ((ConstI32)(uintptr_t)pfx)[g];
+    } else {
+        const unsigned Z = (unsigned)a.tile_zdim, pairs8 = (unsigned)a.tile_groups;
+        const int64_t pair = (int64_t)die + 8 * (int64_t)(a.ride_z ? kk / Z : kk % pairs8);
+        zblock = (int)(a.ride_z ? kk % Z : kk / pairs8);
+        if (pair >= (int64_t)a.nseg * a.H) return;
+        g = (int)(pair / a.H);
+        h = pair % a.H;
+    }
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     const SegRec rec = load_rec(pv.recs, g);
     const int M = rec.M, K = rec.K;
@@ -397,13 +416,24 @@ int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg
     if (info) z = std::min<int64_t>(z, (4 * info->total_rows / std::max<int64_t>(nseg, 1) + round_rows - 1) / round_rows);
     z = std::max<int64_t>(z, 1);
     if (nseg <= 0) return BA_OK;
-    const int64_t pairs8 = (nseg * args.H + 7) / 8;    // pairs per die, rounded up
-    if (pairs8 * z * 8 > 0x7fffffff || pairs8 > 0x7fffffff) return BA_ERR_UNSUPPORTED;
     RunArgs run = args;
-    run.tile_zdim = (int)z;
-    run.tile_groups = (int)pairs8;
-    run.ride_z = (info && info->total_rows >= 512 * nseg) ? 1 : 0;   // tall segments: row blocks of a pair side by side
-    const dim3 grid((unsigned)(pairs8 * z * 8));
+    dim3 grid;
+    if (info && info->total_rows >= 0) {
+        // the batch's totals are known: one workgroup per existing row block (at most total_rows / round_rows
+        // + nseg of them per head), found through the plan's row-block prefix
+        const int64_t items = (info->total_rows / round_rows + nseg) * args.H;
+        const int64_t share = (items + 7) / 8;
+        if (share * 8 > 0x7fffffff) return BA_ERR_UNSUPPORTED;
+        run.ride_slots = 1;
+        grid = dim3((unsigned)(share * 8));
+    } else {
+        const int64_t pairs8 = (nseg * args.H + 7) / 8;    // pairs per die, rounded up
+        if (pairs8 * z * 8 > 0x7fffffff || pairs8 > 0x7fffffff) return BA_ERR_UNSUPPORTED;
+        run.tile_zdim = (int)z;
+        run.tile_groups = (int)pairs8;
+        run.ride_z = 0;
+        grid = dim3((unsigned)(pairs8 * z * 8));
+    }
     if (dtype == BA_F16) { if (qt == 2) launch_nk<0, 2>(nk, grid, stream, run, V); else launch_nk<0, 1>(nk, grid, stream, run, V); }
     else { if (qt == 2) launch_nk<1, 2>(nk, grid, stream, run, V); else launch_nk<1, 1>(nk, grid, stream, run, V); }
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;

@@ -3,7 +3,9 @@
 //
 //   PlanHeader                    (256 bytes)
 //   SegRec recs[cap]              one 48-byte record per segment: offsets and shape
-//   SegRec lists[4][cap]          the records of each launch class once more, compacted (work lists)
+//   SegRec lists[5][cap]          the records of each launch class once more, compacted (work lists)
+//   int32  rowblocks[2][cap + 4]  GEMM plans: exclusive prefix over the segments of their row blocks of 64 and of
+//                                 128 rows (the one-pass attention's work items); entry nseg = all of them
 //
 // cap = nseg rounded up so that every array starts 16-byte aligned.  The
 // compute kernels read the plan through scalar loads (it is never written
@@ -61,8 +63,11 @@ enum PrefixKind {
     kPfxRows = 9,   // softmax: M rows
     kPfxPack = 10,  // 1 for the first segment of a pack of tiny segments, else 0
     kPfxSlow = 11,  // ceil(M/16) for segments the 16-byte operand loads cannot serve
-    kNumPrefix = 12
+    kPfxAtt64 = 12,   // one-pass attention, GEMM plans: ceil(M/64) for segments with rows and a head dimension
+    kPfxAtt128 = 13,  // the same in row blocks of 128
+    kNumPrefix = 14
 };
+constexpr int kAttBlockRows = 64;   // kPfxAtt64 counts blocks of this many rows, kPfxAtt128 of twice as many
 
 // A segment is "aligned" when K % 8 == 0 and its A and B offsets are multiples
 // of 8 elements: every operand row then starts on a 16-byte boundary (given
@@ -136,9 +141,16 @@ struct PlanView {
     SegRec *list[kNumLists];    // records of one launch class, compacted, in segment order
 };
 
+__host__ __device__ inline size_t plan_lists_end(int64_t nseg) {
+    return sizeof(PlanHeader) + (1 + kNumLists) * (size_t)plan_cap(nseg) * sizeof(SegRec);
+}
 __host__ __device__ inline size_t plan_bytes_for(int64_t nseg) {
-    const size_t cap = (size_t)plan_cap(nseg);
-    return sizeof(PlanHeader) + (1 + kNumLists) * cap * sizeof(SegRec);
+    return plan_lists_end(nseg) + 2 * ((size_t)plan_cap(nseg) + 4) * sizeof(int32_t);     // cap is a multiple of 4
+}
+// Row-block prefix `which` (0: blocks of 64 rows, 1: of 128): entry g = blocks of the segments before g,
+// entry nseg = all.
+__host__ __device__ inline int32_t *plan_rowblocks(void *buf, int64_t nseg, int which) {
+    return (int32_t *)((char *)buf + plan_lists_end(nseg)) + (size_t)which * ((size_t)plan_cap(nseg) + 4);
 }
 
 __host__ __device__ inline PlanView plan_view(void *buf, int64_t nseg) {

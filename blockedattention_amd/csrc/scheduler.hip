@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     PlanView pv = plan_view(a.plan, nseg);
 
     int64_t base64[3] = {0, 0, 0};
-    int32_t base32[kNumPrefix] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    int32_t base32[kNumPrefix] = {};
     int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
     int32_t maxSmallN = 0, maxSmallM = 0;       // widest / tallest segment of the strip kernel's main launch
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
@@ -196,6 +196,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         v32[kPfxRows] = ni >= 1 ? mi : 0;
         v32[kPfxPack] = pack > 0 ? 1 : 0;
         v32[kPfxSlow] = aligned ? 0 : strips;
+        const bool att_rows = mi >= 1 && ki >= 1;              // the attention kernel works on these, whatever N is
+        v32[kPfxAtt64] = att_rows ? (mi + kAttBlockRows - 1) / kAttBlockRows : 0;
+        v32[kPfxAtt128] = att_rows ? (mi + 2 * kAttBlockRows - 1) / (2 * kAttBlockRows) : 0;
         if (a.kind == 1) {
 #pragma unroll
             for (int q = 0; q < kNumPrefix; ++q)
@@ -214,6 +217,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             for (int q = 0; q < kNumLists; ++q)          // v32 now holds the exclusive scans
                 if (cls == q) pv.list[q][base32[q] + v32[q]] = rec;
             if (wide_rows) pv.list[kListRows][base32[kListRows] + v32[kListRows]] = rec;
+            if (a.kind == 0) {
+                plan_rowblocks(a.plan, nseg, 0)[g] = base32[kPfxAtt64] + v32[kPfxAtt64];
+                plan_rowblocks(a.plan, nseg, 1)[g] = base32[kPfxAtt128] + v32[kPfxAtt128];
+            }
             if (!offsets_given) {
                 if (a.a1) a.a1[g] = o1;
                 if (a.a2) a.a2[g] = o2;
@@ -274,6 +281,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->small_max_N = rSN; h->small_max_M = rSM;
         h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
         h->run_errors = 0;
+        plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
+        plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
     }
 }
 
