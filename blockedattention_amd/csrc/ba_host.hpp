@@ -15,7 +15,8 @@ enum RunFlags : int {
     kFlagOutF32 = 8,       // fused path writes fp32 probabilities
     kFlagPacksToo = 16,    // strip kernel: the blocks behind its own list walk the pack leaders of the rest list
     kFlagTilesToo = 32,    // strip kernel, 64 KiB launch: further blocks run the tile kernel's workgroups (tile_zdim, tile_groups)
-    kFlagQuiet = 64        // an earlier launch of the same call reports a plan that does not match
+    kFlagQuiet = 64,       // an earlier launch of the same call reports a plan that does not match
+    kFlagSmallToo = 128    // strip kernel, 64 KiB launch: the slots from both_split on walk the main launch's list
 };
 
 struct RunArgs {
@@ -34,6 +35,7 @@ struct RunArgs {
     int tile_groups;  // which take the first tile_groups blocks of a flat grid; the strip part then has
     int ride_slots;   // ride_slots x H x ride_z workgroups, slot fastest
     int ride_z;
+    int both_split;   // with kFlagSmallToo: length of the launch's own list; slot s >= both_split is entry s - both_split of the small list
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,

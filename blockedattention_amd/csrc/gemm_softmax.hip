@@ -689,6 +689,10 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
         bz = lin / ((unsigned)a.ride_slots * (unsigned)a.H);
         gz = (unsigned)a.ride_z;
     }
+    if ((a.flags & kFlagSmallToo) && bx >= (unsigned)a.both_split) {
+        bx -= (unsigned)a.both_split;
+        a.list = kListSmall;
+    }
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     const int64_t h = by;
     // header and record are fetched together; nothing waits on the header alone
@@ -770,10 +774,23 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     const int64_t tile_groups = ceil_div(n_tile, kDies) * kDies * (int64_t)H * tile_z;
     const bool tiles_ride = info && n_big > 0 && n_tile > 0 && tile_groups <= 4096 && (dtype == BA_F16 || dtype == BA_BF16);
     bool tiles_taken = false;
+    // Both strip lists go in ONE launch with the 64 KiB window, the 64 KiB segments first, where two launches
+    // would each be bound by the life of a workgroup rather than by how many are resident: when the main
+    // launch's list holds wide segments (more than eight column tiles: three workgroups per compute unit by
+    // registers, against two in the 64 KiB launch), or when the batch is small (measured: the non-square
+    // 512-segment batch 23.6 -> 19.4 us, the power-law batch 51.2 -> 49.9 us).
+    static const int merge_env = [] { const char *e = getenv("BLOCKEDATTN_MERGE_STRIPS"); return e ? atoi(e) : -1; }();
+    const bool merge = info && n_small > 0 && n_big > 0 &&
+                       (merge_env >= 0 ? merge_env != 0 : info->small_max_N > 128 || (n_small + n_big) * (int64_t)H <= 4096);
     for (int pass = 0; pass < 2; ++pass) {
         int64_t slots = pass == 0 ? n_small : n_big;
-        if (slots <= 0) continue;
+        if (slots <= 0 || (merge && pass == 0)) continue;
         RunArgs fa = args;
+        if (merge) {
+            fa.flags |= kFlagSmallToo;
+            fa.both_split = (int)n_big;
+            slots += n_small;
+        }
         if (packs_ride && !packs_taken) {
             fa.flags |= kFlagPacksToo;
             slots += n_rest;
@@ -791,7 +808,7 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
         fa.list = pass == 0 ? kListSmall : kListBig;
         fa.lds_blocks = pass == 0 ? kFastBlocks : kBigBlocks;
         bool lean_pass = lean;
-        if (info && pass == 0) {
+        if (info && pass == 0 && !merge) {
             // the main launch is sized by ITS widest and tallest segment, not the batch's
             const int64_t nt = fast_strip_tiles((int)std::max(info->small_max_N, 1));
             const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
