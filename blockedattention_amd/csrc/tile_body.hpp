@@ -32,7 +32,7 @@
 // running maximum and a running sum of exp2((s - max) * c) over the lane's own
 // columns (rescaled when the maximum moves); after it the sixteen lanes of a row
 // group are combined once.  Sweep 2 recomputes the scores and writes
-// exp2((s - max) * c) / sum.  The scores never touch memory; the price is the
+// exp2((s - max) * c - log2(sum)): the division rides in the exponent.  The scores never touch memory; the price is the
 // second set of MFMAs, which this memory-bound kernel has room for.
 //
 // Ragged N: the last column chunk is the 128 columns ENDING at N (it overlaps the
@@ -193,7 +193,7 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
         int cbi = 0, slab = 0;                           // chunk being computed
         if (nspan == 1 && active) load_a(0);
 
-        // sweep 1: running maximum and sum of the lane's own columns; sweep 2: -max*c and 1/sum of the row
+        // sweep 1: running maximum and sum of the lane's own columns; sweep 2: m_run = -max*c - log2(sum) of the row
         float m_run[kRT][4], l_run[kRT][4];
 #pragma unroll
         for (int rt = 0; rt < kRT; ++rt)
@@ -317,7 +317,7 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
                 if (overlap && last_chunk) update(std::true_type{});
                 else update(std::false_type{});
                 if (it == per_sweep - 1) {
-                    // combine the sixteen lanes of each row group; leave -max*c and 1/sum for sweep 2
+                    // combine the sixteen lanes of each row group; leave -max*c - log2(sum) for sweep 2
 #pragma unroll
                     for (int rt = 0; rt < kRT; ++rt) {
                         float mx[4], sm[4];
@@ -331,7 +331,7 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
                         }
                         row16_sum4(sm);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) l_run[rt][e] = __builtin_amdgcn_rcpf(sm[e]);
+                        for (int e = 0; e < 4; ++e) m_run[rt][e] -= __builtin_amdgcn_logf(sm[e]);   // 1/sum goes into the exponent
                     }
                 }
                 continue;
@@ -345,8 +345,7 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
                     for (int ct = 0; ct < kCT; ++ct)
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            acc[rt][ct][e] =
-                                __builtin_amdgcn_exp2f(fmaf(acc[rt][ct][e], c, m_run[rt][e])) * l_run[rt][e];
+                            acc[rt][ct][e] = __builtin_amdgcn_exp2f(fmaf(acc[rt][ct][e], c, m_run[rt][e]));
             }
             const uint32_t voff = (uint32_t)((row0 + 4 * rg) * N + cb + 8 * j) * kOutBytes;
 #pragma unroll
