@@ -70,6 +70,42 @@ def blockGEMMSoftmax(
                                                    float(scale), bool(out_fp32))
 
 
+class _FusedAttention(torch.autograd.Function):
+    """Forward: the one-pass kernel.  Backward: the probabilities are recomputed and the gradient taken through
+    the operators the kernel replaces (dV = P^T dO and dP = dO V^T as two blockGEMM calls, dq and dk by the
+    backward passes of blockSoftmax and blockGEMM), so only q, k and v are kept between the passes -- never an
+    ``M x N`` array."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, MList, NList, KList, mat1Accum, mat2Accum, outAccum, scale):
+        out = blockAttention.sparseBlockedAttention(q, k, v, mat1Accum, mat2Accum, outAccum, MList, NList, KList,
+                                                    scale)
+        ctx.save_for_backward(q, k, v)
+        ctx.meta = (MList, NList, KList, mat1Accum, mat2Accum, outAccum)
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        q, k, v = ctx.saved_tensors
+        MList, NList, KList, mat1Accum, mat2Accum, outAccum = ctx.meta
+        if MList is None or NList is None or KList is None:
+            raise RuntimeError("blockFusedAttention: the backward pass needs MList, NList and KList "
+                               "(prefix sums alone do not describe the second product)")
+        grad_out = grad_out.reshape(q.shape[:-1].numel(), -1).contiguous()
+        with torch.enable_grad():
+            qg, kg = (t.detach().requires_grad_(True) for t in (q, k))
+            probs = blockSoftmax(blockGEMM(qg, kg, mat1Accum, mat2Accum, outAccum, MList, NList, KList),
+                                 MList, NList, outAccum, scale=ctx.scale)
+        with torch.no_grad():
+            # dV_g = P_g^T dO_g: N x K, reduction over M, both operands stored reduction-major
+            dv = blockGEMM(probs.detach(), grad_out, None, None, None, NList, KList, MList, True, True)
+            # dP_g = dO_g V_g^T: M x N, reduction over K, both operands row-major
+            dprobs = blockGEMM(grad_out, v.detach(), mat1Accum, mat2Accum, outAccum, MList, NList, KList)
+        dq, dk = torch.autograd.grad(probs, (qg, kg), dprobs)
+        return dq.view_as(q), dk.view_as(k), dv.view_as(v), None, None, None, None, None, None, None
+
+
 def blockFusedAttention(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     MList: Optional[torch.Tensor] = None, NList: Optional[torch.Tensor] = None, KList: Optional[torch.Tensor] = None,
@@ -77,14 +113,17 @@ def blockFusedAttention(
     outAccum: Optional[torch.Tensor] = None,
     scale: float = 1.0,
 ) -> torch.Tensor:
-    """``softmax(scale * Q_g @ K_g^T) @ V_g`` per segment in one pass (forward only).
+    """``softmax(scale * Q_g @ K_g^T) @ V_g`` per segment in one pass.
 
     ``q`` is ``[H, sum(M*K)]`` (the first operand of ``blockGEMM``), ``k`` and ``v`` are both
     ``[H, sum(N*K)]`` (its second operand's layout); the metadata is ``blockGEMM``'s.  The result,
     ``[H, sum(M*K)]``, is what ``blockGEMM(blockSoftmax(blockGEMM(q, k, ...), M, N, scale=scale), v, ...,
     transpose2=True)`` computes, without the ``M x N`` arrays ever reaching memory.  Head dimensions up
-    to 128.
+    to 128.  Differentiable in q, k and v when the size lists are given: the backward pass recomputes the
+    probabilities and runs the backward of that chain.
     """
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _FusedAttention.apply(q, k, v, MList, NList, KList, mat1Accum, mat2Accum, outAccum, float(scale))
     return blockAttention.sparseBlockedAttention(q, k, v, mat1Accum, mat2Accum, outAccum, MList, NList, KList,
                                                  float(scale))
 

@@ -126,3 +126,42 @@ def test_head_dimension_above_128_is_refused(dev):
     t = torch.zeros((1, 4 * 136), dtype=torch.float16, device=dev)
     with pytest.raises(RuntimeError, match="unsupported"):
         capi.varlen_attention(plan, t, t, t, torch.empty_like(t), 1, 4 * 136, 4 * 136, 16, 1.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_backward_matches_per_segment_autograd(dev, dtype):
+    # dq, dk, dv of the one-pass operator against torch.autograd on the per-segment fp32 oracle (same 16-bit
+    # inputs).  The backward rounds the recomputed scores and probabilities, dP, dS and the results to the
+    # 16-bit type (u = 2^-11 / 2^-9 each), and dS = P (dP - sum P dP) cancels: the bound is that of the scores,
+    # |g - ref| <= tol (|ref| + rms(ref)), with tol = 20 u (1e-2 for fp16, 4e-2 for bf16).
+    import blockedAttention
+    M = [50, 120, 8, 33]; N = [64, 33, 200, 7]; K = [64, 64, 64, 64]
+    Q, Km, V = operands(M, N, K, 2, dtype, seed=9, sigma=0.5)
+    Md, Nd, Kd = (torch.tensor(x, dtype=torch.int64, device=dev) for x in (M, N, K))
+    q, k, v = (t.to(dev).requires_grad_() for t in (Q, Km, V))
+    out = blockedAttention.blockFusedAttention(q, k, v, Md, Nd, Kd, scale=0.125)
+    g = torch.Generator(device="cpu").manual_seed(10)
+    wgt = torch.randn(out.shape, generator=g).to(dtype)
+    out.backward(wgt.to(dev))
+    qr, kr, vr = (t.float().requires_grad_() for t in (Q, Km, V))
+    ref = oracle.per_segment_torch_attention(qr, kr, vr, M, N, K, 0.125)
+    ref.backward(wgt.float())
+    tol = 1e-2 if dtype == torch.float16 else 4e-2
+    for name, got, want in (("dq", q.grad, qr.grad), ("dk", k.grad, kr.grad), ("dv", v.grad, vr.grad)):
+        assert got.dtype == dtype and got.shape == want.shape
+        got = got.float().cpu()
+        assert not torch.isnan(got).any(), name
+        rms = float(want.pow(2).mean().sqrt())
+        excess = (got - want).abs() - (tol * want.abs() + tol * rms)
+        assert excess.max().item() <= 0, f"{name}: off by {float((got - want).abs().max())} (rms {rms})"
+
+
+def test_backward_needs_the_size_lists(dev):
+    import blockedAttention
+    M = np.array([4, 9]); N = np.array([5, 3]); K = np.array([8, 8])
+    a1, a2, ao = (torch.from_numpy(x).to(dev) for x in oracle.lists_to_accum(M, N, K))
+    q = torch.randn((1, int((M * K).sum())), device=dev, dtype=torch.float16, requires_grad=True)
+    kv = torch.randn((1, int((N * K).sum())), device=dev, dtype=torch.float16)
+    out = blockedAttention.blockFusedAttention(q, kv, kv, mat1Accum=a1, mat2Accum=a2, outAccum=ao)
+    with pytest.raises(RuntimeError, match="MList"):
+        out.sum().backward()
