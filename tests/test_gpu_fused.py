@@ -115,3 +115,24 @@ def test_launches_without_the_host_summary(dev):
         plan = run_all(dev, M, N, K, 2, dtype, scale, seed=5, summary=False)
         i = plan.info
         assert i.list_big == 1 and i.list_tile == 4 and i.list_rows == 2 and i.pack_items == 1
+
+
+def test_both_strip_lists_merged_and_separate(dev):
+    # Segments for both LDS windows of the strip kernel (B_g up to 32 KiB / up to 64 KiB), packs and tile-kernel
+    # segments in one batch.  Few (list entry, head) pairs, or wide segments in the 32 KiB list: one launch takes
+    # both lists.  Many pairs and a narrow 32 KiB list: one launch per list.
+    rng = np.random.default_rng(21)
+    def batch(nseg, wide_small):
+        M = rng.integers(1, 40, nseg); K = np.full(nseg, 128)
+        N = np.where(rng.random(nseg) < 0.8, rng.integers(2, 129, nseg), rng.integers(129, 257, nseg))
+        if wide_small:
+            K[:8] = 32; N[:8] = 250                      # 16 tiles x 1 k-step: the 32 KiB list, wider than 128
+        N[-1] = 300; M[-1] = 130                         # one tile-kernel segment rides along
+        return M, N, K
+    for nseg, heads, wide_small in ((40, 2, False), (40, 2, True), (600, 7, False), (600, 7, True)):
+        M, N, K = batch(nseg, wide_small)
+        plan = run_all(dev, M, N, K, heads, torch.bfloat16, 0.09, seed=nseg + heads, check_softmax=False)
+        i = plan.info
+        assert i.list_small > 0 and i.list_big > 0 and i.list_tile == 1
+        assert (i.small_max_N > 128) == wide_small
+        assert ((i.list_small + i.list_big) * heads > 4096) == (nseg == 600)
