@@ -337,15 +337,13 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void at
     if (!header_ok(a)) { report_mismatch(a); return; }
     // Workgroup -> (segment, head, row block).  Consecutive workgroup ids go to the eight dies of the chip in
     // turn, and each die has its own L2: id = die + 8 k.  All row blocks of one (segment, head) pair read the
-    // same keys and values, so they get consecutive k on ONE die (pair = die + 8 (k / Z), row block k % Z) and
-    // run at about the same time; with the head as the fast index of a pair, every die gets its share of
-    // every segment.
-    // (Short segments, where most pairs have fewer row blocks than Z and nothing to share: row block as the
-    // slow index instead, ride_z = 0, so that the workgroups that find no rows come last.)
+    // same keys and values, so they should run on ONE die at about the same time.
     // With the row-block prefix (ride_slots = 1, launches that know the batch's totals): the existing
     // (head, segment, row block) items, head-major, are cut into eight contiguous shares, one per die, so the
-    // row blocks of a pair still sit side by side on one die and no workgroup is launched for a row block that
-    // does not exist, except past the end of a share (the grid is sized from an upper bound of the item count).
+    // row blocks of a pair sit side by side on one die and no workgroup is launched for a row block that does
+    // not exist, except past the end of a share (the grid is sized from an upper bound of the item count).
+    // Without it: pair = die + 8 (k mod pairs per die), row block k / pairs per die; a workgroup takes every
+    // tile_zdim-th row block of its pair, and the workgroups that find no rows come last.
     const unsigned id = blockIdx.x, die = id & 7u, kk = id >> 3;
     int g, zblock;
     int64_t h;
@@ -354,15 +352,18 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void at
         const int64_t per_head = ((ConstI32)(uintptr_t)pfx)[a.nseg];
         const int64_t items = per_head * a.H, share = (items + 7) >> 3;
         const int64_t u = (int64_t)die * share + kk;
+        // a grid too small for the plan's items: the host summary the launch was sized from is not this plan's
+        if (id == 0 && threadIdx.x == 0 && share * 8 > (int64_t)gridDim.x)
+            atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         if (kk >= share || u >= items) return;
         h = u / per_head;
         const int item = (int)(u % per_head);
         g = prefix_search(pfx, a.nseg, item);
         zblock = item - ((ConstI32)(uintptr_t)pfx)[g];
     } else {
-        const unsigned Z = (unsigned)a.tile_zdim, pairs8 = (unsigned)a.tile_groups;
-        const int64_t pair = (int64_t)die + 8 * (int64_t)(a.ride_z ? kk / Z : kk % pairs8);
-        zblock = (int)(a.ride_z ? kk % Z : kk / pairs8);
+        const unsigned pairs8 = (unsigned)a.tile_groups;
+        const int64_t pair = (int64_t)die + 8 * (int64_t)(kk % pairs8);
+        zblock = (int)(kk / pairs8);
         if (pair >= (int64_t)a.nseg * a.H) return;
         g = (int)(pair / a.H);
         h = pair % a.H;
@@ -383,7 +384,8 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void at
 
 template <int DT, int QT>
 static void launch_nk(int nk, dim3 grid, hipStream_t stream, const RunArgs &args, const void *V) {
-    // args.tile_zdim = row blocks per (segment, head) pair, tile_groups = pairs per die, ride_z = row block fastest
+    // args.ride_slots = 1: work items from the plan's row-block prefix; else args.tile_zdim = row blocks per
+    // (segment, head) pair, tile_groups = pairs per die
     switch (nk) {
         case 1: hipLaunchKernelGGL((attention_kernel<DT, 1, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
         case 2: hipLaunchKernelGGL((attention_kernel<DT, 2, QT>), grid, dim3(kAttThreads), 0, stream, args, V); break;
@@ -431,7 +433,6 @@ int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg
         if (pairs8 * z * 8 > 0x7fffffff || pairs8 > 0x7fffffff) return BA_ERR_UNSUPPORTED;
         run.tile_zdim = (int)z;
         run.tile_groups = (int)pairs8;
-        run.ride_z = 0;
         grid = dim3((unsigned)(pairs8 * z * 8));
     }
     if (dtype == BA_F16) { if (qt == 2) launch_nk<0, 2>(nk, grid, stream, run, V); else launch_nk<0, 1>(nk, grid, stream, run, V); }
