@@ -757,11 +757,15 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     const int64_t n_tile = !mfma_ok ? 0 : info ? info->list_tile : nseg;
     const int64_t n_rest = !mfma_ok ? nseg : info ? info->list_rest : nseg;
     const bool lean = info && info->max_N <= 128;
-    // z: enough workgroups to fill the machine, at most one per kSegWaves strips of the tallest segment
-    auto strip_z = [&](int64_t slots, int64_t tallest) {
+    // z: enough workgroups to fill the machine, at most one per kSegWaves strips of the tallest segment.  The
+    // narrow build (up to eight column tiles, four to five workgroups resident per compute unit) aims at eight
+    // workgroups per compute unit; the wide build holds two (64 KiB window) or three (registers), and one round of
+    // resident workgroups that loop over their strips beats several rounds of short ones (non-square 512-segment
+    // batch: 17.9 us with one workgroup per segment, 19.7 us with four).
+    auto strip_z = [&](int64_t slots, int64_t tallest, int per_cu) {
         if (!info) return (int64_t)2;
         const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(tallest, 1), kStripRows), kSegWaves);
-        const int64_t want = ceil_div((int64_t)cus * 8, std::max<int64_t>(1, slots * (int64_t)H));
+        const int64_t want = ceil_div((int64_t)cus * per_cu, std::max<int64_t>(1, slots * (int64_t)H));
         return std::max<int64_t>(1, std::min<int64_t>(groups, std::min<int64_t>(want, 64)));
     };
     // the rest list is nothing but pack leaders: the first strip launch takes them along
@@ -802,7 +806,7 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
             fa.tile_zdim = (int)tile_z;
             fa.tile_groups = (int)tile_groups;
             fa.ride_slots = (int)slots;
-            fa.ride_z = (int)strip_z(slots, info->max_M);
+            fa.ride_z = (int)strip_z(slots, info->max_M, 2);
             tiles_taken = true;
         }
         fa.list = pass == 0 ? kListSmall : kListBig;
@@ -816,7 +820,7 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
             lean_pass = info->small_max_N <= 128;
         }
         const int64_t tallest = !info ? 0 : pass == 0 ? info->small_max_M : info->max_M;
-        const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots, tallest));
+        const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots, tallest, lean_pass ? 8 : pass == 0 ? 3 : 2));
         // room for the copy of the ragged run behind the image of B_g, while the total stays within 64 KiB
         fa.lds_extra = fa.lds_blocks * kLdsBlockBytes + kRaggedCopyBytes <= 65536 ? kRaggedCopyBytes : 0;
         const size_t lds_bytes = (size_t)fa.lds_blocks * kLdsBlockBytes + fa.lds_extra;
