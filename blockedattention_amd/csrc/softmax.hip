@@ -20,6 +20,7 @@
 //                    the eight columns 8*l + 512*k; rows of up to 4096 columns stay
 //                    in registers, longer rows are re-read in three passes.
 #include <algorithm>
+#include <cstdlib>
 
 #include "ba_gemm_common.hpp"
 
@@ -198,18 +199,18 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
 // MAXG = 8 is the build for batches whose widest row has 128 columns or fewer: half the registers,
 // twice the resident wavefronts.
 template <int DT, bool BACKWARD, int MAXG>
-__global__ __launch_bounds__(kSoftmaxThreads, MAXG <= 8 ? 3 : 1) void softmax_runs_kernel(SoftmaxArgs a) {
+__device__ __forceinline__ void softmax_runs_body(const SoftmaxArgs &a, unsigned bx, unsigned by, unsigned bz, unsigned gz) {
     typedef typename Io<DT>::T T;
     const int nseg = softmax_plan_nseg(a);
-    const int g = blockIdx.x;
+    const int g = bx;
     if (g >= nseg) return;
     const PlanRO pv = plan_ro(a.plan, nseg);
     const SegRec rec = load_rec(pv.recs, g);
     const int rows = rec.M, cols = rec.N;
     if (cols < 1 || cols > kRunCols || cols > 16 * MAXG || rows < 1) return;
     const int wave = uniform((int)(threadIdx.x >> 6));
-    const int first = blockIdx.z * kSoftmaxWaves + wave, step = gridDim.z * kSoftmaxWaves;
-    const int64_t seg0 = (int64_t)blockIdx.y * a.Dsrc + rec.offO;
+    const int first = bz * kSoftmaxWaves + wave, step = gz * kSoftmaxWaves;
+    const int64_t seg0 = (int64_t)by * a.Dsrc + rec.offO;
     if (cols == 1) {
         // one column: softmax is 1 (NaN where the input is not finite); backward is 0 * (...) likewise
         const T *src = reinterpret_cast<const T *>(a.src) + seg0;
@@ -333,8 +334,14 @@ __device__ __forceinline__ void softmax_rows_forward(const typename Io<DT>::T *s
     }
 }
 
+template <int DT, bool BACKWARD, int MAXG>
+__global__ __launch_bounds__(kSoftmaxThreads, MAXG <= 8 ? 3 : 1) void softmax_runs_kernel(SoftmaxArgs a) {
+    softmax_runs_body<DT, BACKWARD, MAXG>(a, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z);
+}
+
+// lin = linear index of the workgroup in a grid of (list entries, gy heads, gz row groups)
 template <int DT, bool BACKWARD>
-__global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxArgs a) {
+__device__ __forceinline__ void softmax_rows_body(const SoftmaxArgs &a, uint64_t lin, unsigned gy, unsigned gz) {
     typedef typename Io<DT>::T T;
     // walks the plan's list of wide segments: the grid is as long as the list (or longer, without a host
     // copy of the plan summary)
@@ -346,16 +353,15 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
     // then the head, then the list entry makes the machine work through one (segment, head) after the
     // other, each as one stream of consecutive rows; with the entry fastest it would read and write
     // hundreds of segments of unequal row lengths at once, which costs a third of the bandwidth.
-    const uint64_t lin = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
-    const unsigned group = (unsigned)(lin % gridDim.z), head = (unsigned)((lin / gridDim.z) % gridDim.y);
-    const unsigned entry = (unsigned)(lin / ((uint64_t)gridDim.z * gridDim.y));
+    const unsigned group = (unsigned)(lin % gz), head = (unsigned)((lin / gz) % gy);
+    const unsigned entry = (unsigned)(lin / ((uint64_t)gz * gy));
     const SegRec rec = load_rec(pv.recs + (int64_t)(kListRows + 1) * plan_cap(nseg), entry);
     if ((int)entry >= count) return;
     const int rows = rec.M, cols = rec.N;
     if (cols <= kRunCols) return;                       // the lane-run kernel's
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int lane = lane_id();
-    const int first = group * kSoftmaxWaves + wave, stride = gridDim.z * kSoftmaxWaves;
+    const int first = group * kSoftmaxWaves + wave, stride = gz * kSoftmaxWaves;
     const int64_t seg0 = (int64_t)head * a.Dsrc + rec.offO;
     const T *src = reinterpret_cast<const T *>(a.src) + seg0;
     const T *aux = reinterpret_cast<const T *>(a.aux) + seg0;
@@ -466,6 +472,30 @@ __global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxAr
 }
 
 template <int DT, bool BACKWARD>
+__global__ __launch_bounds__(kSoftmaxThreads) void softmax_rows_kernel(SoftmaxArgs a) {
+    const uint64_t lin = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
+    softmax_rows_body<DT, BACKWARD>(a, lin, gridDim.y, gridDim.z);
+}
+
+// Both kernels in one launch (flat grid): the first both.rows_blocks workgroups are the row kernel's (wide
+// rows run longest, so they start first), the rest decode to the lane-run kernel's (segment, head, row group),
+// segment fastest.  Two launches that would each leave part of the machine idle become one.
+struct BothGrid {
+    unsigned rows_blocks, rows_z, runs_slots, runs_z;
+};
+template <int DT>
+__global__ __launch_bounds__(kSoftmaxThreads, 3) void softmax_both_kernel(SoftmaxArgs a, BothGrid both) {
+    const unsigned id = blockIdx.x;
+    if (id < both.rows_blocks) {
+        softmax_rows_body<DT, false>(a, id, (unsigned)a.H, both.rows_z);
+        return;
+    }
+    const unsigned r = id - both.rows_blocks;
+    const unsigned bx = r % both.runs_slots, by = (r / both.runs_slots) % (unsigned)a.H;
+    softmax_runs_body<DT, false, 16>(a, bx, by, r / (both.runs_slots * (unsigned)a.H), both.runs_z);
+}
+
+template <int DT, bool BACKWARD>
 static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
     if (args.H > 65535) return BA_ERR_UNSUPPORTED;      // heads ride on gridDim.y
     const int cus = device_cu_count();
@@ -489,6 +519,20 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
     }
     if (nseg <= 0) return BA_OK;
     const dim3 grid_runs((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs);
+    if constexpr (!BACKWARD) {
+        // a modest row-kernel launch (it would not fill the machine for long) rides with the lane-run kernel
+        static const int both_env = [] { const char *e = getenv("BLOCKEDATTN_SOFTMAX_BOTH"); return e ? atoi(e) : -1; }();
+        const int64_t rows_blocks = n_rows * args.H * z_rows, runs_blocks = nseg * args.H * z_runs;
+        const bool both = info && rows_work && n_rows < nseg && info->max_N > 128 &&
+                          rows_blocks + runs_blocks < (int64_t(1) << 31) &&
+                          (both_env >= 0 ? both_env != 0 : rows_blocks <= (int64_t)cus * 64);
+        if (both) {
+            const BothGrid bg{(unsigned)rows_blocks, (unsigned)z_rows, (unsigned)nseg, (unsigned)z_runs};
+            hipLaunchKernelGGL((softmax_both_kernel<DT>), dim3((unsigned)(rows_blocks + runs_blocks)), dim3(kSoftmaxThreads), 0,
+                               stream, args, bg);
+            return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+        }
+    }
     if (info && info->max_N <= 128)
         hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 8>), grid_runs, dim3(kSoftmaxThreads), 0, stream, args);
     else
