@@ -194,6 +194,21 @@ __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t v) {
     v += dpp64_or_zero<0x143, 0xc>(v);
     return v;
 }
+// Inclusive scan inside every row of 16 lanes (four independent scans per wavefront).
+__device__ __forceinline__ int row16_inclusive_scan(int v) {
+    v += dpp_or_zero<0x111, 0xf>(v);
+    v += dpp_or_zero<0x112, 0xf>(v);
+    v += dpp_or_zero<0x114, 0xf>(v);
+    v += dpp_or_zero<0x118, 0xf>(v);
+    return v;
+}
+__device__ __forceinline__ int64_t row16_inclusive_scan(int64_t v) {
+    v += dpp64_or_zero<0x111, 0xf>(v);
+    v += dpp64_or_zero<0x112, 0xf>(v);
+    v += dpp64_or_zero<0x114, 0xf>(v);
+    v += dpp64_or_zero<0x118, 0xf>(v);
+    return v;
+}
 // Maximum of non-negative ints over the wavefront (result in every lane).
 __device__ __forceinline__ int wave_max_nonneg(int v) {
     v = max(v, dpp_or_zero<0x111, 0xf>(v));

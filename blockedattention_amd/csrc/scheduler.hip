@@ -28,27 +28,47 @@ struct SchedArgs {
 };
 
 // Exclusive scan of NQ quantities over the workgroup.  Wavefront-level DPP
-// scans, then the 16 wavefront totals are scanned by lanes 0..15 of every
-// wavefront (one row of DPP shifts).  lds holds NQ * kSchedWaves entries and
-// is free for reuse after the next __syncthreads().  One barrier.
+// scans; the totals of the (up to 16) wavefronts go to LDS as lds[16 q + wavefront] and are scanned four
+// quantities at a time: lane l of every wavefront takes entry 64 b + l of batch b, i.e. quantity 4 b + l / 16 of
+// wavefront l % 16, and one scan inside the rows of 16 lanes serves all four.  lds holds 16 * NQ entries and is
+// free for reuse after the next __syncthreads().  One barrier (none in the one-wavefront build).
 template <typename T, int NQ, int kSchedWaves>
 __device__ __forceinline__ void block_exclusive_scan(T (&v)[NQ], T (&total)[NQ], T *lds) {
+    static_assert(kSchedWaves <= 16, "one row of 16 lanes scans the wavefront totals");
     const int wave = uniform((int)(threadIdx.x >> 6)), lane = lane_id();
     T incl[NQ];
+    if constexpr (kSchedWaves == 1) {
+        // one wavefront: its own scan is the workgroup's (callers still place their barrier before reusing lds)
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            incl[q] = wave_inclusive_scan(v[q]);
+            total[q] = readlane_t(incl[q], 63);
+            v[q] = incl[q] - v[q];
+        }
+        return;
+    }
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
         incl[q] = wave_inclusive_scan(v[q]);
-        if (lane == 63) lds[q * kSchedWaves + wave] = incl[q];
+        if (lane == 63) lds[q * 16 + wave] = incl[q];
     }
     __syncthreads();
+    constexpr int kBatches = (NQ + 3) / 4;
+    const bool mine = (lane & 15) < kSchedWaves;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-        T t = lane < kSchedWaves ? lds[q * kSchedWaves + lane] : T(0);
-        t = wave_inclusive_scan(t);                    // lanes 0..15 now hold the scan over wavefronts
-        const T upto = readlane_t(t, kSchedWaves - 1);
-        const T before = wave == 0 ? T(0) : readlane_t(t, wave - 1);
-        v[q] = before + incl[q] - v[q];
-        total[q] = upto;
+    for (int b = 0; b < kBatches; ++b) {
+        T t = (mine && 64 * b + lane < 16 * NQ) ? lds[64 * b + lane] : T(0);
+        t = row16_inclusive_scan(t);                   // lanes 16 r .. 16 r + 15: scan over wavefronts of quantity 4 b + r
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int q = 4 * b + r;
+            if (q < NQ) {
+                const T upto = readlane_t(t, 16 * r + kSchedWaves - 1);
+                const T before = wave == 0 ? T(0) : readlane_t(t, 16 * r + wave - 1);
+                v[q] = before + incl[q] - v[q];
+                total[q] = upto;
+            }
+        }
     }
 }
 
@@ -85,8 +105,8 @@ __device__ __forceinline__ bool derive_lists(int64_t mk, int64_t nk, int64_t mn,
 template <int kSchedThreads>
 __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     constexpr int kSchedWaves = kSchedThreads / 64;
-    __shared__ int64_t sScan64[kSchedWaves * 3];
-    __shared__ int32_t sScan32[kSchedWaves * kNumPrefix];
+    __shared__ int64_t sScan64[16 * 3];
+    __shared__ int32_t sScan32[16 * kNumPrefix];
     __shared__ int32_t sRed[kSchedWaves][6];
 
     const int tid = threadIdx.x;
