@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         int32_t pack = 0;
         // Only batches that contain segments small enough to pack pay for the window walk.
         const bool packable = aligned && mi >= 1 && ni >= 1 && ki >= 1 && mi < kPackDim && ni < kPackDim;
-        if (a.kind == 0 && __syncthreads_or(packable)) {
+        if (a.kind == 0 && __ballot(packable) != 0) {          // per wavefront: the windows are rows of 16 lanes
             // A window is the 16 lanes of one DPP row.  The greedy walk runs along the row: lane j takes the
             // state that lane j-1 holds (rows sum, columns sum, members so far, K of the open pack), decides
             // whether its segment joins that pack, and holds the state after it.  After step t lanes 0..t
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
 #pragma unroll
             for (int q = 0; q < 3; ++q) base64[q] += t64[q];
         }
-        if (nseg == 0) break;
+        if (chunk + kSchedThreads >= nseg) break;
         __syncthreads();   // the scan scratch is rewritten by the next pass
     }
 
