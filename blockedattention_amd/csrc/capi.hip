@@ -75,10 +75,18 @@ __attribute__((visibility("default"))) int ba_plan_softmax(void *plan, size_t pl
 
 __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_plan_info *info, ba_stream_t stream) {
     if (!plan || !info) return BA_ERR_INVALID_ARG;
-    PlanHeader h;
-    if (hipMemcpyAsync(&h, plan, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+    // The header lands in pinned host memory (one 256-byte buffer per calling thread, allocated at the thread's
+    // first call and kept for the life of the process): the copy then needs no staging by the runtime.
+    static thread_local PlanHeader *pinned = [] {
+        void *p = nullptr;
+        return hipHostMalloc(&p, sizeof(PlanHeader), hipHostMallocDefault) == hipSuccess ? (PlanHeader *)p : nullptr;
+    }();
+    PlanHeader on_stack;
+    PlanHeader *dst = pinned ? pinned : &on_stack;
+    if (hipMemcpyAsync(dst, plan, sizeof(PlanHeader), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
         return BA_ERR_LAUNCH;
     if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return BA_ERR_LAUNCH;
+    const PlanHeader h = *dst;
     if (h.magic != kPlanMagic) return BA_ERR_INVALID_ARG;
     memset(info, 0, sizeof(*info));
     info->nseg = h.nseg;

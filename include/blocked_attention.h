@@ -111,8 +111,10 @@ int ba_plan_softmax(void *plan, size_t plan_bytes, int64_t nseg,
                     int64_t *accum, int accum_given, ba_stream_t stream);
 
 /* Copies the plan summary to the host and waits for it (the one blocking
- * call).  Returns BA_ERR_BAD_METADATA if the scheduler rejected any segment
- * or a kernel refused to run against the plan.
+ * call, and the one that allocates: 256 bytes of pinned host memory at a
+ * thread's first call, kept for the life of the process, through which the
+ * summary travels).  Returns BA_ERR_BAD_METADATA if the scheduler rejected any
+ * segment or a kernel refused to run against the plan.
  *
  * The compute entry points below take `nseg` (the segment count the plan was
  * built for; it sizes the launch grids) and the summary as `info` (a HOST
