@@ -484,7 +484,7 @@ struct BothGrid {
     unsigned rows_blocks, rows_z, runs_slots, runs_z;
 };
 template <int DT>
-__global__ __launch_bounds__(kSoftmaxThreads, 3) void softmax_both_kernel(SoftmaxArgs a, BothGrid both) {
+__global__ __launch_bounds__(kSoftmaxThreads, DT == 2 ? 2 : 3) void softmax_both_kernel(SoftmaxArgs a, BothGrid both) {
     const unsigned id = blockIdx.x;
     if (id < both.rows_blocks) {
         softmax_rows_body<DT, false>(a, id, (unsigned)a.H, both.rows_z);
