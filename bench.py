@@ -316,6 +316,19 @@ def main():
             steps = args.steps if cfg != 5 else max(5, min(args.steps, 20))
             f = c.gpu_figures(steps, min(args.warmup, steps), with_unfused=cfg != 5)
             f["parity_max_abs_err"] = err
+            if cfg == 1 and not args.no_cpu:
+                # the reference's own CPU-runnable case, on the host: the scalar C restatement (one core) and the
+                # per-segment torch path (all cores), fp32, median of 20 runs
+                import oracle
+                A32, B32 = c.A_host.float().numpy(), c.B_host.float().numpy()
+                def med(fn, n=20):
+                    ts = []
+                    for _ in range(n):
+                        t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
+                    return round(sorted(ts)[n // 2] * 1e6, 1)
+                f["cpu_c_port_us"] = med(lambda: oracle.gemm_softmax(A32, B32, c.w.M, c.w.N, c.w.K, c.w.scale))
+                f["cpu_torch_us"] = med(lambda: oracle.per_segment_torch(c.A_host.float(), c.B_host.float(), c.w.M, c.w.N,
+                                                                         c.w.K, c.w.scale))
             others[f"cfg{cfg}"] = f
             del c
             torch.cuda.empty_cache()
