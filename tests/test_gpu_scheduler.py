@@ -163,3 +163,27 @@ def test_row_block_prefixes_of_the_attention_work_list(dev):
             want = np.concatenate([[0], np.cumsum(blocks)]).astype(np.int32)
             got = words[which * (cap + 4): which * (cap + 4) + nseg + 1]
             assert np.array_equal(got, want), (nseg, rows)
+
+
+def test_main_strip_list_is_a_permutation_in_work_buckets(dev):
+    # Batches of 65 to 256 segments keep the main strip launch's list in eight buckets of decreasing work
+    # (16-row strips x column tiles / 8, clipped at 7), in segment order inside a bucket; every other batch
+    # keeps segment order.  Either way the list holds each of its segments exactly once.
+    rec = np.dtype([("o1", "<i8"), ("o2", "<i8"), ("oo", "<i8"), ("M", "<i4"), ("N", "<i4"), ("K", "<i4"),
+                    ("pack", "<i4"), ("kind", "<i4"), ("index", "<i4")])
+    rng = np.random.default_rng(5)
+    for nseg in (40, 200, 256, 300):
+        M = rng.integers(17, 130, nseg); N = rng.integers(17, 130, nseg); K = np.full(nseg, 64)
+        plan = make_plan(dev, M, N, K)
+        assert plan.info.list_small == nseg
+        cap = (nseg + 4) & ~3
+        raw = plan.buf.cpu().numpy()
+        lst = raw[256 + cap * 48: 256 + cap * 48 + nseg * 48].view(rec)
+        assert sorted(lst["index"].tolist()) == list(range(nseg))
+        assert np.array_equal(lst["M"], M[lst["index"]]) and np.array_equal(lst["N"], N[lst["index"]])
+        bucket = np.minimum(7, ((M + 15) // 16) * (2 * ((N + 31) // 32)) // 8)
+        if 64 < nseg <= 256:
+            want = np.argsort(-bucket, kind="stable")
+        else:
+            want = np.arange(nseg)
+        assert np.array_equal(lst["index"], want), nseg
