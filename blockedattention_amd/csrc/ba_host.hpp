@@ -16,7 +16,8 @@ enum RunFlags : int {
     kFlagPacksToo = 16,    // strip kernel: the blocks behind its own list walk the pack leaders of the rest list
     kFlagTilesToo = 32,    // strip kernel, 64 KiB launch: further blocks run the tile kernel's workgroups (tile_zdim, tile_groups)
     kFlagQuiet = 64,       // an earlier launch of the same call reports a plan that does not match
-    kFlagSmallToo = 128    // strip kernel, 64 KiB launch: the slots from both_split on walk the main launch's list
+    kFlagSmallToo = 128,   // strip kernel, 64 KiB launch: the slots from both_split on walk the main launch's list
+    kFlagHeadFast = 256    // strip kernel: grid (head, slot, z) instead of (slot, head, z)
 };
 
 struct RunArgs {

@@ -63,6 +63,7 @@ struct SoftmaxArgs {
     void *dst;           // forward: y            backward: dx
     int64_t H, Dsrc;
     float scale;
+    int head_fast;       // lane-run kernel: grid (head, segment, z) instead of (segment, head, z)
 };
 
 // Plan checks shared by both kernels, fetched as one batch of scalar loads.
@@ -336,7 +337,8 @@ __device__ __forceinline__ void softmax_rows_forward(const typename Io<DT>::T *s
 
 template <int DT, bool BACKWARD, int MAXG>
 __global__ __launch_bounds__(kSoftmaxThreads, MAXG <= 8 ? 3 : 1) void softmax_runs_kernel(SoftmaxArgs a) {
-    softmax_runs_body<DT, BACKWARD, MAXG>(a, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z);
+    if (a.head_fast) softmax_runs_body<DT, BACKWARD, MAXG>(a, blockIdx.y, blockIdx.x, blockIdx.z, gridDim.z);
+    else softmax_runs_body<DT, BACKWARD, MAXG>(a, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z);
 }
 
 // lin = linear index of the workgroup in a grid of (list entries, gy heads, gz row groups)
@@ -491,7 +493,8 @@ __global__ __launch_bounds__(kSoftmaxThreads, DT == 2 ? 2 : 3) void softmax_both
         return;
     }
     const unsigned r = id - both.rows_blocks;
-    const unsigned bx = r % both.runs_slots, by = (r / both.runs_slots) % (unsigned)a.H;
+    const unsigned bx = a.head_fast ? (r / (unsigned)a.H) % both.runs_slots : r % both.runs_slots;
+    const unsigned by = a.head_fast ? r % (unsigned)a.H : (r / both.runs_slots) % (unsigned)a.H;
     softmax_runs_body<DT, false, 16>(a, bx, by, r / (both.runs_slots * (unsigned)a.H), both.runs_z);
 }
 
@@ -520,7 +523,13 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
                                                         (info->max_M + kSoftmaxWaves - 1) / kSoftmaxWaves));
     }
     if (nseg <= 0) return BA_OK;
-    const dim3 grid_runs((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs);
+    // head as the fastest grid index of the lane-run kernel: workgroups that start together are the heads of one
+    // segment and take equally long
+    static const int hf = [] { const char *e = getenv("BLOCKEDATTN_HEAD_FAST"); return e ? atoi(e) : 1; }();
+    SoftmaxArgs run = args;
+    run.head_fast = hf && nseg <= 65535 ? 1 : 0;
+    const dim3 grid_runs = run.head_fast ? dim3((unsigned)args.H, (unsigned)nseg, (unsigned)z_runs)
+                                         : dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z_runs);
     if constexpr (!BACKWARD) {
         // a modest row-kernel launch (it would not fill the machine for long) rides with the lane-run kernel
         static const int both_env = [] { const char *e = getenv("BLOCKEDATTN_SOFTMAX_BOTH"); return e ? atoi(e) : -1; }();
@@ -531,14 +540,14 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
         if (both) {
             const BothGrid bg{(unsigned)rows_blocks, (unsigned)z_rows, (unsigned)nseg, (unsigned)z_runs};
             hipLaunchKernelGGL((softmax_both_kernel<DT>), dim3((unsigned)(rows_blocks + runs_blocks)), dim3(kSoftmaxThreads), 0,
-                               stream, args, bg);
+                               stream, run, bg);
             return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
         }
     }
     if (info && info->max_N <= 128)
-        hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 8>), grid_runs, dim3(kSoftmaxThreads), 0, stream, args);
+        hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 8>), grid_runs, dim3(kSoftmaxThreads), 0, stream, run);
     else
-        hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 16>), grid_runs, dim3(kSoftmaxThreads), 0, stream, args);
+        hipLaunchKernelGGL((softmax_runs_kernel<DT, BACKWARD, 16>), grid_runs, dim3(kSoftmaxThreads), 0, stream, run);
     if (rows_work)
         hipLaunchKernelGGL((softmax_rows_kernel<DT, BACKWARD>),
                            dim3((unsigned)n_rows, (unsigned)args.H, (unsigned)z_rows), dim3(kSoftmaxThreads), 0, stream,
