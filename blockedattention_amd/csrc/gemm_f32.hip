@@ -27,7 +27,8 @@ constexpr int kF32PitchA = kF32K + 4;                // 16-byte rows, staggered 
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-// grid (segment, head, z): workgroup z takes the 64-row rounds z, z + gridDim.z, ... of its segment.
+// grid (head, segment, z) with kFlagHeadFast (consecutive workgroups, which go to the dies in turn, are the heads
+// of one segment), else (segment, head, z): workgroup z takes the 64-row rounds z, z + gridDim.z, ... of its segment.
 __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
     __shared__ float sB[kF32Cols * kF32PitchB];
     __shared__ __attribute__((aligned(16))) float sA[kF32Waves][kStripRows * kF32PitchA];
@@ -40,7 +41,8 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
             atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
     }
-    const int g = blockIdx.x;
+    const bool head_fast = a.flags & kFlagHeadFast;
+    const int g = head_fast ? blockIdx.y : blockIdx.x;
     if (g >= nseg) return;
     const PlanRO pv = plan_ro(a.plan, nseg);
     const SegRec rec = load_rec(pv.recs, g);
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(kF32Threads) void gemm_f32_kernel(RunArgs a) {
     const int wave = uniform(tid >> 6);
     const int lane = lane_id();
     const bool t1 = a.flags & kFlagTranspose1, t2 = a.flags & kFlagTranspose2;
-    const int64_t h = blockIdx.y;
+    const int64_t h = head_fast ? blockIdx.x : blockIdx.y;
     const float *as = reinterpret_cast<const float *>(a.A) + h * a.Dm1 + rec.off1;
     const float *bs = reinterpret_cast<const float *>(a.B) + h * a.Dm2 + rec.off2;
     float *os = reinterpret_cast<float *>(a.out) + h * a.Dout + rec.offO;
@@ -150,8 +152,12 @@ int launch_gemm_f32(const RunArgs &args, int64_t nseg, const ba_plan_info *info,
         z = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(rounds, want), 64));
     }
     if (nseg <= 0) return BA_OK;
-    hipLaunchKernelGGL(gemm_f32_kernel, dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z), dim3(kF32Threads), 0,
-                       stream, args);
+    RunArgs run = args;
+    const bool head_fast = nseg <= 65535;               // segments then ride on gridDim.y
+    if (head_fast) run.flags |= kFlagHeadFast;
+    hipLaunchKernelGGL(gemm_f32_kernel,
+                       head_fast ? dim3((unsigned)args.H, (unsigned)nseg, (unsigned)z) : dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z),
+                       dim3(kF32Threads), 0, stream, run);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 

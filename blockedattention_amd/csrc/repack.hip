@@ -38,6 +38,7 @@ struct RepackArgs {
     int nseg;
     int src_which, dst_which; // 0: A (M x K), 1: B (N x K), 2: out (M x N)
     int swap_dims, column_major;
+    int head_fast;            // grid (head, segment, z): consecutive workgroups are the heads of one segment
 };
 
 __device__ __forceinline__ void operand_of(const SegRec &r, int which, int &rows, int &cols, int64_t &off) {
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(kRepackThreads) void repack_kernel(RepackArgs a) {
             atomicAdd(&reinterpret_cast<PlanHeader *>(const_cast<void *>(a.dst_plan))->run_errors, 1);
         return;
     }
-    const int g = blockIdx.x;
+    const int g = a.head_fast ? blockIdx.y : blockIdx.x;
     if (g >= a.nseg) return;
     const SegRec rs = load_rec(plan_ro(const_cast<void *>(a.src_plan), a.nseg).recs, g);
     const SegRec rd = load_rec(plan_ro(const_cast<void *>(a.dst_plan), a.nseg).recs, g);
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(kRepackThreads) void repack_kernel(RepackArgs a) {
     operand_of(rs, a.src_which, Rs, Cs, offs);
     if (a.swap_dims) { const int t = Rs; Rs = Cs; Cs = t; }
     if (R < 1 || C < 1) return;
-    const int64_t h = blockIdx.y;
+    const int64_t h = a.head_fast ? blockIdx.x : blockIdx.y;
     const uint16_t *src = a.src + h * a.Dsrc + offs;
     uint16_t *dst = a.dst + h * a.Ddst + offd;
     const int tid = threadIdx.x;
@@ -164,8 +165,10 @@ int launch_repack(const void *src_plan, int src_which, int swap_dims, int column
         z = std::max<int64_t>(1, std::min<int64_t>(z, 1024));
     }
     RepackArgs a{src_plan, dst_plan, (const uint16_t *)src, (uint16_t *)dst, Dsrc, Ddst, (int)nseg,
-                 src_which, dst_which, swap_dims, column_major};
-    hipLaunchKernelGGL(repack_kernel, dim3((unsigned)nseg, (unsigned)H, (unsigned)z), dim3(kRepackThreads), 0, stream, a);
+                 src_which, dst_which, swap_dims, column_major, nseg <= 65535 ? 1 : 0};
+    hipLaunchKernelGGL(repack_kernel,
+                       a.head_fast ? dim3((unsigned)H, (unsigned)nseg, (unsigned)z) : dim3((unsigned)nseg, (unsigned)H, (unsigned)z),
+                       dim3(kRepackThreads), 0, stream, a);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
