@@ -28,3 +28,18 @@ def test_random_batches(dev, seed):
     sigma = 0.3 if int(Ks.max()) > 100 else 1.0                     # keeps fp16 scores far from overflow
     run_all(dev, M, N, Ks, H, dtype, scale, seed=seed, sigma=sigma)
     run_all(dev, M, N, Ks, H, dtype, scale, seed=seed + 50, sigma=sigma, summary=False)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_batches_of_65_to_256_segments(dev, seed):
+    # the scheduler build that keeps the main strip list in work buckets; head counts that are not powers of two
+    rng = np.random.default_rng(300 + seed)
+    nseg = int(rng.integers(65, 257))
+    Ks = rng.choice([64, 128, 32, 72, 8], nseg, p=[0.4, 0.3, 0.1, 0.1, 0.1]).astype(np.int64)
+    N = rng.integers(1, 260, nseg).astype(np.int64)
+    M = rng.integers(1, 150, nseg).astype(np.int64)
+    N[:3] = [300, 1, 16]; M[:3] = [40, 5, 3]
+    H = int(rng.choice([1, 3, 5, 8, 9]))
+    dtype = torch.float16 if seed % 2 else torch.bfloat16
+    run_all(dev, M, N, Ks, H, dtype, 0.1, seed=seed, sigma=0.3)
+    run_all(dev, M, N, Ks, H, dtype, 0.1, seed=seed + 50, sigma=0.3, summary=False)
