@@ -1,4 +1,4 @@
-"""Scheduler + fused pair recorded into a HIP graph: the device-side scheduler lets a replay pick up a
+"""Scheduler, GEMM, softmax, fused pair and one-pass attention recorded into a HIP graph: the device-side scheduler lets a replay pick up a
 new segmentation (same totals) without the host reading anything back."""
 import numpy as np
 import pytest
@@ -23,6 +23,7 @@ def test_graph_replays_follow_the_lists_on_the_device(dev):
     A = torch.empty((H, d1), dtype=dtype, device=dev); B = torch.empty_like(A)
     scores = torch.empty((H, do), dtype=dtype, device=dev); probs = torch.empty_like(scores)
     fused = torch.empty_like(scores)
+    V = torch.empty_like(B); att = torch.empty_like(A)
     plan = capi.Plan(40, dev)
 
     def record():
@@ -30,6 +31,7 @@ def test_graph_replays_follow_the_lists_on_the_device(dev):
         capi.varlen_gemm(plan, A, B, scores, H, d1, d1, do)
         capi.blocked_softmax(plan, scores, probs, H, do, scale)
         capi.gemm_softmax(plan, A, B, fused, H, d1, d1, do, scale)
+        capi.varlen_attention(plan, A, B, V, att, H, d1, d1, do, scale)
 
     record()                                                   # eager once (lazy initialisation outside capture)
     torch.cuda.synchronize()
@@ -42,6 +44,8 @@ def test_graph_replays_follow_the_lists_on_the_device(dev):
         Ah, Bh = random_operands(m, m, K, H, dtype, seed=10 + replay)
         Md.copy_(dev_i64(m, dev)); Nd.copy_(Md)
         A.copy_(Ah); B.copy_(Bh)
+        Vh = random_operands(m, m, K, H, dtype, seed=30 + replay)[1]
+        V.copy_(Vh); att.fill_(float("nan"))
         scores.fill_(float("nan")); probs.fill_(float("nan")); fused.fill_(float("nan"))
         junk = torch.randn(1 << 20, device=dev).sum()          # the program's own eager work between replays
         torch.cuda.synchronize()
@@ -51,6 +55,7 @@ def test_graph_replays_follow_the_lists_on_the_device(dev):
         assert_scores_close(scores, sc, f"replay {replay} scores")
         assert_probs_close(fused, pr, f"replay {replay} fused")
         assert_probs_close(probs, oracle.per_segment_torch_softmax(scores.cpu(), m, m, scale), f"replay {replay} softmax")
+        assert_scores_close(att, oracle.per_segment_torch_attention(Ah, Bh, Vh, m, m, K, scale), f"replay {replay} attention")
         assert torch.equal(ao.cpu(), torch.as_tensor(oracle.lists_to_accum(m, m, K)[2]))
         assert float(junk) == float(junk)
     assert plan.read().run_errors == 0
