@@ -136,3 +136,13 @@ def test_both_strip_lists_merged_and_separate(dev):
         assert i.list_small > 0 and i.list_big > 0 and i.list_tile == 1
         assert (i.small_max_N > 128) == wide_small
         assert ((i.list_small + i.list_big) * heads > 4096) == (nseg == 600)
+
+
+def test_more_list_entries_than_the_second_grid_dimension_holds(dev):
+    # 66 000 strip-class segments: the list entries cannot ride on gridDim.y (65 535 at most), so the launches
+    # fall back to the entry as the fastest grid index; the scheduler takes 65 passes.
+    rng = np.random.default_rng(8)
+    nseg = 66000
+    M = rng.integers(17, 25, nseg); N = rng.integers(17, 25, nseg); K = np.full(nseg, 8)
+    plan = run_all(dev, M, N, K, 2, torch.float16, 0.3, seed=2)
+    assert plan.info.list_small == nseg
