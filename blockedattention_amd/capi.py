@@ -18,8 +18,9 @@ META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
 SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
     "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax", "ba_repack_operand",
-    "ba_varlen_attention",
+    "ba_varlen_attention", "ba_gemm_softmax_static",
 )
+STATIC_MAX_SEGMENTS = 4096   # BA_STATIC_MAX_SEGMENTS
 
 
 class PlanInfo(ctypes.Structure):
@@ -80,6 +81,8 @@ def load():
     lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
     lib.ba_varlen_attention.restype = i32
     lib.ba_varlen_attention.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, vp, i64, i64, i64, i64, f32, vp]
+    lib.ba_gemm_softmax_static.restype = i32
+    lib.ba_gemm_softmax_static.argtypes = [i64, i32, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
     _lib = lib
     return lib
 
@@ -197,6 +200,18 @@ def gemm_softmax(plan, A, B, out, H, Dm1, Dm2, Dout, scale=1.0):
     st = load().ba_gemm_softmax(plan.ptr, plan._hint(), plan.nseg, dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out),
                                 dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
     check(st, "ba_gemm_softmax")
+    return out
+
+
+def gemm_softmax_static(MList, NList, KList, A, B, out, H, Dm1, Dm2, Dout, scale=1.0, accum1=None, accum2=None,
+                        accumOut=None, mode=META_FROM_LISTS):
+    """Scheduler + fused pair with the plan in the library's own device buffer (see ba_gemm_softmax_static):
+    no allocation, no read-back."""
+    nseg = MList.numel() if MList is not None else accumOut.numel() - 1
+    st = load().ba_gemm_softmax_static(nseg, mode, _ptr(MList), _ptr(NList), _ptr(KList), _ptr(accum1), _ptr(accum2),
+                                       _ptr(accumOut), dtype_code(A.dtype), _ptr(A), _ptr(B), _ptr(out),
+                                       dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
+    check(st, "ba_gemm_softmax_static")
     return out
 
 

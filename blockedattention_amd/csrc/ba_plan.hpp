@@ -91,7 +91,7 @@ struct PlanHeader {
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 
-__host__ __device__ inline int64_t plan_cap(int64_t nseg) { return (nseg + 4) & ~int64_t(3); }
+__host__ __device__ constexpr int64_t plan_cap(int64_t nseg) { return (nseg + 4) & ~int64_t(3); }
 
 // How a segment is processed.
 enum SegKind : int32_t {
@@ -141,10 +141,10 @@ struct PlanView {
     SegRec *list[kNumLists];    // records of one launch class, compacted, in segment order
 };
 
-__host__ __device__ inline size_t plan_lists_end(int64_t nseg) {
+__host__ __device__ constexpr size_t plan_lists_end(int64_t nseg) {
     return sizeof(PlanHeader) + (1 + kNumLists) * (size_t)plan_cap(nseg) * sizeof(SegRec);
 }
-__host__ __device__ inline size_t plan_bytes_for(int64_t nseg) {
+__host__ __device__ constexpr size_t plan_bytes_for(int64_t nseg) {
     return plan_lists_end(nseg) + 2 * ((size_t)plan_cap(nseg) + 4) * sizeof(int32_t);     // cap is a multiple of 4
 }
 // Row-block prefix `which` (0: blocks of 64 rows, 1: of 128): entry g = blocks of the segments before g,

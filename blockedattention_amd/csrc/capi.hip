@@ -3,9 +3,32 @@
 // except ba_plan_read.
 #include <string.h>
 
+#include <mutex>
+
 #include "ba_host.hpp"
 
+// Plan buffer of ba_gemm_softmax_static: one array per GPU the library runs on, held until the process ends.
+// In host code the name is only a handle for hipGetSymbolAddress; kernels and launch arguments get the
+// address that call returns for the current device.
+constexpr size_t kStaticPlanBytes = (ba::plan_bytes_for(BA_STATIC_MAX_SEGMENTS) + 255) & ~size_t(255);
+static __device__ __align__(256) unsigned char scratch[kStaticPlanBytes];
+
 namespace ba {
+
+// Device address of `scratch` on the current device, looked up once per device.
+static void *static_plan_buffer() {
+    static std::mutex lock;
+    static void *ptr[64] = {nullptr};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        ptr[dev] = p;
+    }
+    return ptr[dev];
+}
 
 int device_cu_count() {
     static int cached[64] = {0};
@@ -177,6 +200,31 @@ __attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_
     args.flags |= mfma_flag(args);
     if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
     return launch_strips(dtype, 1, args, nseg, info, (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_gemm_softmax_static(int64_t nseg, int mode, int64_t *MList,
+                                                                  int64_t *NList, int64_t *KList, int64_t *accum1,
+                                                                  int64_t *accum2, int64_t *accumOut, int dtype,
+                                                                  const void *A, const void *B, void *out,
+                                                                  int out_dtype, int64_t H, int64_t Dm1, int64_t Dm2,
+                                                                  int64_t Dout, float scale, ba_stream_t stream) {
+    if (nseg < 0 || bad_sizes(H, Dm1, Dm2, Dout)) return BA_ERR_INVALID_ARG;
+    if (nseg > BA_STATIC_MAX_SEGMENTS) return BA_ERR_WORKSPACE;
+    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
+    if (out_dtype != dtype && out_dtype != BA_F32) return BA_ERR_UNSUPPORTED;
+    void *plan = static_plan_buffer();
+    if (!plan) return BA_ERR_LAUNCH;
+    // The scheduler rewrites the whole header (run-error counter included), every record and every list entry
+    // a kernel can reach, so nothing of the previous call's plan is read.
+    const int st = launch_schedule(plan, kStaticPlanBytes, nseg, mode, 0, MList, NList, KList, accum1, accum2, accumOut,
+                                   (hipStream_t)stream);
+    if (st != BA_OK) return st;
+    if (H == 0 || Dout == 0 || nseg == 0) return BA_OK;
+    if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
+    RunArgs args{plan, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, 0, (int)nseg};
+    args.flags |= mfma_flag(args);
+    if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
+    return launch_strips(dtype, 1, args, nseg, nullptr, (hipStream_t)stream);
 }
 
 __attribute__((visibility("default"))) int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg,

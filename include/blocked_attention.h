@@ -212,6 +212,28 @@ int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg, int 
                         const void *V, void *out, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout, float scale,
                         ba_stream_t stream);
 
+/*
+ * ba_gemm_softmax for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  Scheduler and fused pair in one
+ * call: the plan lives in a buffer that is part of the library's device image
+ * (one copy per GPU, held until the process ends), so the caller passes only
+ * the metadata (mode and pointers as for ba_plan_gemm), operands and output.
+ * Nothing is allocated and nothing is read back: the kernels take their work
+ * lists from the plan on the device, exactly as ba_gemm_softmax does with
+ * info == NULL, and give the same results.  Metadata the scheduler rejects
+ * leaves `out` unwritten (there is no summary to report it through), so check
+ * new metadata once with ba_plan_gemm + ba_plan_read.
+ * At most BA_STATIC_MAX_SEGMENTS segments: more returns BA_ERR_WORKSPACE.
+ * All calls on one GPU share that GPU's buffer: calls that overlap on one GPU
+ * (different streams or threads) race; calls on one stream do not.
+ */
+#define BA_STATIC_MAX_SEGMENTS 4096
+int ba_gemm_softmax_static(int64_t nseg, int mode, int64_t *MList, int64_t *NList, int64_t *KList,
+                           int64_t *accum1, int64_t *accum2, int64_t *accumOut, int dtype, const void *A,
+                           const void *B, void *out, int out_dtype, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
+                           float scale, ba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
