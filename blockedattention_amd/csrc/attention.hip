@@ -421,9 +421,10 @@ int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg
     RunArgs run = args;
     dim3 grid;
     if (info && info->total_rows >= 0) {
-        // the batch's totals are known: one workgroup per existing row block (at most total_rows / round_rows
-        // + nseg of them per head), found through the plan's row-block prefix
-        const int64_t items = (info->total_rows / round_rows + nseg) * args.H;
+        // the batch's totals are known: one workgroup per existing row block, found through the plan's
+        // row-block prefix (segments without keys count: their output rows are zeroed)
+        const int64_t items = (int64_t)(qt == 2 ? info->att_blocks128 : info->att_blocks64) * args.H;
+        if (items <= 0) return BA_OK;
         const int64_t share = (items + 7) / 8;
         if (share * 8 > 0x7fffffff) return BA_ERR_UNSUPPORTED;
         run.ride_slots = 1;

@@ -87,7 +87,8 @@ struct PlanHeader {
     int32_t bad_segments;
     int32_t run_errors;      // bumped by kernels that refuse to run
     int32_t small_max_N, small_max_M;   // maxima over the segments of the strip kernel's main launch
-    int32_t pad_[21];
+    int32_t att_blocks64, att_blocks128;   // totals of kPfxAtt64 / kPfxAtt128: the one-pass attention's row blocks per head
+    int32_t pad_[19];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 

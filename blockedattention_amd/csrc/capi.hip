@@ -131,6 +131,8 @@ __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_pla
     info->list_rows = (int32_t)h.totals[kListRows];
     info->small_max_N = h.small_max_N;
     info->small_max_M = h.small_max_M;
+    info->att_blocks64 = h.att_blocks64;
+    info->att_blocks128 = h.att_blocks128;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 

@@ -328,6 +328,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->small_max_N = rSN; h->small_max_M = rSM;
         h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
         h->run_errors = 0;
+        h->att_blocks64 = base32[kPfxAtt64];
+        h->att_blocks128 = base32[kPfxAtt128];
         plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
         plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
     }

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BA_ABI_VERSION 1
+#define BA_ABI_VERSION 2
 
 typedef void *ba_stream_t; /* hipStream_t */
 
@@ -55,7 +55,7 @@ typedef enum ba_meta_mode {
 typedef struct ba_plan_info {
     int64_t nseg;
     int64_t Dm1, Dm2, Dout; /* last prefix-sum entries = elements per head */
-    int64_t total_rows;     /* sum of M */
+    int64_t total_rows;     /* rows of the softmax: sum of M over the segments with N >= 1 */
     /* work-item totals (16-row strips) by segment shape */
     int64_t gemm_items;     /* 16 x <=256 output pieces of segments with N > 256 */
     int64_t strip_items;    /* 16-row strips of aligned segments with N <= 256 */
@@ -74,6 +74,9 @@ typedef struct ba_plan_info {
     int32_t small_max_N;    /* widest segment of the strip kernel's main launch */
     int32_t small_max_M;    /* tallest segment of the strip kernel's main launch */
     int32_t list_rows;      /* softmax row kernel: segments with N > 256 (GEMM and softmax plans) */
+    /* one-pass attention, GEMM plans: row blocks of 64 and of 128 rows per head, summed over the segments
+     * with M >= 1 and K >= 1 whatever their N (a segment without keys still has its output rows zeroed) */
+    int32_t att_blocks64, att_blocks128;
 } ba_plan_info;
 
 const char *ba_status_string(int status);

@@ -78,6 +78,18 @@ def test_empty_segments_and_no_keys(dev):
     assert torch.equal(out[:, 64:64 + 9 * 24].cpu(), torch.zeros(2, 9 * 24, dtype=torch.float16))
 
 
+def test_tall_segment_without_keys_among_others(dev):
+    # A tall N = 0 segment has row blocks of its own (zeros to write): the launch is sized from the plan's
+    # row-block totals, which count it, so neither its rows nor its neighbours' are left unwritten.
+    M = [64, 1000, 64]; N = [64, 0, 64]; K = [64, 64, 64]
+    for dtype in (torch.float16, torch.bfloat16):
+        out, ref = run(dev, M, N, K, 8, dtype, 0.125)
+        assert torch.equal(out[:, 64 * 64:64 * 64 + 1000 * 64].cpu(), torch.zeros(8, 1000 * 64, dtype=dtype))
+    plan = make_plan(dev, M, N, K)
+    assert plan.info.att_blocks64 == 1 + 16 + 1 and plan.info.att_blocks128 == 1 + 8 + 1
+    assert plan.info.total_rows == 128
+
+
 def test_negative_and_zero_scale(dev):
     M = [9, 70]; N = [100, 17]; K = [16, 64]
     for scale in (-0.3, 0.0):
