@@ -49,6 +49,10 @@ int launch_strips(int dtype, int fused, const RunArgs &args, int64_t nseg, const
 // The tile kernel over the large segments (see tile_segment()); slots = length of its work list (or nseg).
 int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                  hipStream_t stream);
+// The row-block kernel over the same list (large segments, K <= 128, 16-bit output): whole-line stores.
+// BA_ERR_UNSUPPORTED when the plan summary is missing or does not fit; the caller then takes launch_tiles.
+int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
+                     hipStream_t stream);
 int launch_gemm_f32(const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,
                    float scale, const ba_plan_info *info, hipStream_t stream);

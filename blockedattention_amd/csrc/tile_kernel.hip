@@ -20,6 +20,9 @@ static void launch_one(const RunArgs &args, unsigned groups, int zdim, hipStream
 // dimension covers the tallest segment; without it the workgroups loop over row blocks.
 int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                  hipStream_t stream) {
+    static const int use_rowblocks = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK"); return e ? atoi(e) : 1; }();
+    if (use_rowblocks && info && info->max_K <= 128 && !(args.flags & kFlagOutF32))
+        return launch_rowblocks(dtype, fused, args, slots, info, stream);
     int64_t z = 4;
     if (info)
         z = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kTileRows - 1) / kTileRows));

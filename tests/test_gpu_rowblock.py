@@ -1,0 +1,93 @@
+"""Large segments with K <= 128 (the row-block kernel: 256 rows per workgroup, 64 columns at a time, results
+through an LDS ring into line-aligned stores) against the oracle: every line phase, ragged rows and columns,
+every reduction length, the overflow path of the first sweep, GEMM alone and fused."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blockedattention_amd import capi
+from _util import assert_probs_close, assert_scores_close, make_plan, random_operands, run_all
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_shapes_and_phases(dev, dtype):
+    # odd and even widths (rows then start at every 2-byte phase of a 128-byte line), widths around the chunk
+    # and ring sizes, heights around the workgroup's 256 rows and a wavefront's 32, one row, K from 8 to 128
+    M = [300, 256, 257, 1, 40, 33, 513, 31]; N = [257, 300, 1000, 5000, 320, 321, 263, 384]
+    K = [64, 128, 8, 40, 96, 104, 120, 32]
+    plan = run_all(dev, M, N, K, 3, dtype, 0.11, seed=7)
+    assert plan.info.list_tile == len(M)
+
+
+def test_every_width_modulo_the_chunk(dev):
+    # N mod 64 = 0..63 at two sizes: the ragged last chunk, the window behind it and the unaligned end pieces
+    N = np.concatenate([np.arange(257, 321), [448, 449, 511, 512, 513]]); M = np.full(N.size, 37); K = np.full(N.size, 16)
+    run_all(dev, M, N, K, 1, torch.float16, 0.3, seed=3, check_softmax=False)
+    run_all(dev, M[::7], N[::7], K[::7], 2, torch.bfloat16, -0.2, seed=4, check_softmax=False)
+
+
+def test_negative_and_zero_scale_large(dev):
+    for scale in (-0.3, 0.0):
+        run_all(dev, [70, 290], [700, 333], [64, 128], 2, torch.float16, scale, check_gemm=False)
+
+
+def test_scores_far_above_the_first_chunk(dev):
+    # The first sweep measures every score against the row maximum of the FIRST 64 columns.  Here the later
+    # columns exceed it by far more than the exponent range: the sums overflow, and the workgroup repeats the
+    # sweep with a running maximum.  Rows of a second segment in the same call take the fast path.
+    M = np.array([100, 64]); N = np.array([700, 300]); K = np.array([128, 64])
+    A, B = random_operands(M, N, K, 2, torch.float16, seed=11)
+    A = A.abs() + 1; B = B.abs()
+    Bs = B[:, :700 * 128].reshape(2, 700, 128)
+    Bs[:, :64] *= 0.01                                        # tiny scores in the first chunk
+    Bs[:, 300:310] *= 4                                       # the rows' maxima, hundreds above
+    plan = make_plan(dev, M, N, K)
+    i = plan.info
+    out = torch.full((2, i.Dout), float("nan"), dtype=torch.float16, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, 2, i.Dm1, i.Dm2, i.Dout, 1.0)
+    ref = oracle.per_segment_torch(A, B, M, N, K, 1.0)
+    assert_probs_close(out, ref, "overflow path")
+    assert float(out[:, :100 * 700].float().max()) > 0.05     # sharply peaked rows, as constructed
+    assert plan.read().run_errors == 0
+
+
+def test_unaligned_output_base_and_many_heads(dev):
+    # the result tensor starts 2 bytes past a 256-byte boundary and Dout is odd: every head has its own phases
+    M = np.array([131, 50]); N = np.array([259, 641]); K = np.array([64, 64])
+    H = 5
+    A, B = random_operands(M, N, K, H, torch.bfloat16, seed=5)
+    plan = make_plan(dev, M, N, K)
+    i = plan.info
+    assert i.Dout % 2 == 1
+    buf = torch.full((H * i.Dout + 1,), float("nan"), dtype=torch.bfloat16, device=dev)
+    out = buf[1:].view(H, i.Dout)
+    assert out.data_ptr() % 4 == 2
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, H, i.Dm1, i.Dm2, i.Dout, 0.125)
+    assert_probs_close(out, oracle.per_segment_torch(A, B, M, N, K, 0.125), "unaligned base")
+    assert torch.isnan(buf[0])                                 # nothing written in front of the result
+    sc = torch.full((H * i.Dout + 1,), float("nan"), dtype=torch.bfloat16, device=dev)
+    capi.varlen_gemm(plan, A.to(dev), B.to(dev), sc[1:].view(H, i.Dout), H, i.Dm1, i.Dm2, i.Dout)
+    assert_scores_close(sc[1:].view(H, i.Dout), oracle.per_segment_torch(A, B, M, N, K, 0.125, want="both")[0], "scores")
+    assert torch.isnan(sc[0])
+
+
+def test_gaps_between_segments_stay_untouched(dev):
+    # prefix sums given with gaps: the elements between two segments' results keep what they held
+    M = np.array([40, 70]); N = np.array([300, 260]); K = np.array([32, 32])
+    A, B = random_operands(M, N, K, 1, torch.float16, seed=6)
+    a1 = np.array([0, 40 * 32, 40 * 32 + 70 * 32]); a2 = np.array([0, 300 * 32, 300 * 32 + 260 * 32])
+    ao = np.array([0, 40 * 300 + 37, 40 * 300 + 37 + 70 * 260 + 5])
+    from _util import dev_i64
+    plan = capi.plan_gemm(2, dev, dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev), dev_i64(a1, dev), dev_i64(a2, dev),
+                          dev_i64(ao, dev), mode=capi.META_GIVEN)
+    plan.read()
+    out = torch.full((1, int(ao[-1])), 7.0, dtype=torch.float16, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, 1, int(a1[-1]), int(a2[-1]), int(ao[-1]), 0.2)
+    ref = oracle.per_segment_torch(A, B, M, N, K, 0.2)
+    got = out.cpu()
+    assert_probs_close(got[:, :40 * 300], ref[:, :40 * 300], "first")
+    assert_probs_close(got[:, ao[1]:ao[1] + 70 * 260], ref[:, 40 * 300:], "second")
+    assert (got[:, 40 * 300:ao[1]] == 7).all() and (got[:, ao[1] + 70 * 260:] == 7).all()
