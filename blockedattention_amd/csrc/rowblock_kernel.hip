@@ -465,8 +465,12 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                         // window stores of those iterations (each behind its iteration's fill) may stay in flight
                         int later = 0;
 #pragma unroll
-                        for (int k = 1; k <= kRbStages - 2; ++k)
-                            if (it + k < total) later += kRbFillInsts;
+                        for (int k = 1; k <= kRbStages - 2; ++k) {
+                            // (the fill of a ragged last chunk is not counted: its instructions for rows past N
+                            // are skipped altogether, so fewer than kRbFillInsts may have been issued)
+                            const int c = it + k, last = c == ncb - 1 || c == 2 * ncb - 1;
+                            if (c < total && !((N & (kRbCols - 1)) != 0 && last)) later += kRbFillInsts;
+                        }
                         if (active) {
                             const int first_store = (FUSED ? ncb : 0) + 1;    // first iteration whose body stores (interior chunks: 4 instructions)
 #pragma unroll
