@@ -12,7 +12,7 @@ import torch
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libblockedattn_hip.so")
 
-BA_F16, BA_BF16, BA_F32 = 0, 1, 2
+BA_F16, BA_BF16, BA_F32, BA_F64, BA_U8, BA_I8, BA_I16, BA_I32, BA_I64 = range(9)
 META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
 
 SYMBOLS = (
@@ -94,7 +94,9 @@ def check(status, what):
 
 def dtype_code(dtype):
     try:
-        return {torch.float16: BA_F16, torch.bfloat16: BA_BF16, torch.float32: BA_F32}[dtype]
+        return {torch.float16: BA_F16, torch.bfloat16: BA_BF16, torch.float32: BA_F32, torch.float64: BA_F64,
+                torch.uint8: BA_U8, torch.int8: BA_I8, torch.int16: BA_I16, torch.int32: BA_I32,
+                torch.int64: BA_I64}[dtype]
     except KeyError:
         raise BlockedAttentionError(f"unsupported dtype {dtype}") from None
 

@@ -148,7 +148,7 @@ __attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_p
     if (transpose1) args.flags |= kFlagTranspose1;
     if (transpose2) args.flags |= kFlagTranspose2;
     args.flags |= mfma_flag(args);
-    if (dtype == BA_F32) return launch_gemm_f32(args, nseg, info, (hipStream_t)stream);
+    if (dtype != BA_F16 && dtype != BA_BF16) return launch_gemm_generic(dtype, args, nseg, info, (hipStream_t)stream);
     return launch_strips(dtype, 0, args, nseg, info, (hipStream_t)stream);
 }
 

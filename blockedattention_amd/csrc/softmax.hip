@@ -1,7 +1,7 @@
 // Standalone blocked row softmax: dst row = softmax(scale * src row) for every
 // row of every segment (csrc/cuda/spBlkSoftmax.cu:88-138, 182-269 restated for
-// wave64), and its backward.  fp32 arithmetic for every dtype, one rounding at
-// the store, no column limit.
+// wave64), and its backward.  fp32 arithmetic for fp16, bf16 and fp32, one rounding at
+// the store, no column limit; fp64 has a plain kernel of its own at the end of the file.
 //
 // A segment is a contiguous run of rows x cols elements, rows back to back.  The
 // memory pipeline works per lane access, so both kernels move 16 bytes per lane
@@ -555,6 +555,75 @@ static int launch_softmax_t(const SoftmaxArgs &args, int64_t nseg, const ba_plan
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 
+// ---------------------------------------------------------------- fp64
+// The reference instantiates its softmax for double as well (csrc/cuda/spBlkSoftmax.cu:400).  One wavefront per
+// row, arithmetic in double, the row read again for each of the three steps (maximum, sum, result); grid
+// (segment, head, z), wavefront w of workgroup z takes rows 4 z + w, then on in steps of 4 gridDim.z.
+__device__ __forceinline__ double wave_max_f64(double v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmax(v, __shfl_xor(v, m));
+    return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
+template <bool BACKWARD>
+__global__ __launch_bounds__(kSoftmaxThreads) void softmax_f64_kernel(SoftmaxArgs a) {
+    const int nseg = softmax_plan_nseg(a);
+    const int g = blockIdx.x;
+    if (g >= nseg) return;
+    const PlanRO pv = plan_ro(a.plan, nseg);
+    const SegRec rec = load_rec(pv.recs, g);
+    const int rows = rec.M, cols = rec.N;
+    if (rows < 1 || cols < 1) return;
+    const int wave = uniform((int)(threadIdx.x >> 6)), lane = lane_id();
+    const int64_t seg0 = (int64_t)blockIdx.y * a.Dsrc + rec.offO;
+    const double *src = reinterpret_cast<const double *>(a.src) + seg0;
+    const double *aux = reinterpret_cast<const double *>(a.aux) + seg0;
+    double *dst = reinterpret_cast<double *>(a.dst) + seg0;
+    const double scale = (double)a.scale;
+    for (int r = blockIdx.z * kSoftmaxWaves + wave; r < rows; r += gridDim.z * kSoftmaxWaves) {
+        const double *x = src + (int64_t)r * cols;
+        double *y = dst + (int64_t)r * cols;
+        if constexpr (!BACKWARD) {
+            double m = -INFINITY;
+            for (int c = lane; c < cols; c += 64) m = fmax(m, x[c] * scale);
+            m = wave_max_f64(m);
+            double sum = 0.0;
+            for (int c = lane; c < cols; c += 64) sum += exp(x[c] * scale - m);
+            sum = wave_sum_f64(sum);
+            for (int c = lane; c < cols; c += 64) y[c] = exp(x[c] * scale - m) / sum;       // a row of -inf: NaN, like torch
+        } else {
+            const double *dy = aux + (int64_t)r * cols;
+            double dot = 0.0;
+            for (int c = lane; c < cols; c += 64) dot += x[c] * dy[c];
+            dot = wave_sum_f64(dot);
+            for (int c = lane; c < cols; c += 64) y[c] = scale * (dy[c] - dot) * x[c];
+        }
+    }
+}
+
+template <bool BACKWARD>
+static int launch_softmax_f64(const SoftmaxArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
+    if (args.H > 65535) return BA_ERR_UNSUPPORTED;
+    int64_t z = 8;
+    if (info) {
+        nseg = info->nseg;
+        const int64_t pairs = std::max<int64_t>(1, nseg * args.H);
+        const int64_t want = ((int64_t)device_cu_count() * 16 + pairs - 1) / pairs;
+        z = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, 4096),
+                                                   (info->max_M + kSoftmaxWaves - 1) / kSoftmaxWaves));
+    }
+    if (nseg <= 0) return BA_OK;
+    if (nseg > 2147483647) return BA_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((softmax_f64_kernel<BACKWARD>), dim3((unsigned)nseg, (unsigned)args.H, (unsigned)z),
+                       dim3(kSoftmaxThreads), 0, stream, args);
+    return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+}
+
 int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,
                    float scale, const ba_plan_info *info, hipStream_t stream) {
     SoftmaxArgs args{plan, src, nullptr, dst, H, Dsrc, scale};
@@ -562,6 +631,7 @@ int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *d
         case BA_F16: return launch_softmax_t<BA_F16, false>(args, nseg, info, stream);
         case BA_BF16: return launch_softmax_t<BA_BF16, false>(args, nseg, info, stream);
         case BA_F32: return launch_softmax_t<BA_F32, false>(args, nseg, info, stream);
+        case BA_F64: return launch_softmax_f64<false>(args, nseg, info, stream);
         default: return BA_ERR_UNSUPPORTED;
     }
 }
@@ -575,6 +645,7 @@ int launch_softmax_backward(int dtype, void *plan, int64_t nseg, const void *y, 
         case BA_F16: return launch_softmax_t<BA_F16, true>(args, nseg, info, stream);
         case BA_BF16: return launch_softmax_t<BA_BF16, true>(args, nseg, info, stream);
         case BA_F32: return launch_softmax_t<BA_F32, true>(args, nseg, info, stream);
+        case BA_F64: return launch_softmax_f64<true>(args, nseg, info, stream);
         default: return BA_ERR_UNSUPPORTED;
     }
 }

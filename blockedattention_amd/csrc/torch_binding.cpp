@@ -50,7 +50,13 @@ int dtype_code(const Tensor &t, const char *name) {
         case at::kHalf: return BA_F16;
         case at::kBFloat16: return BA_BF16;
         case at::kFloat: return BA_F32;
-        default: TORCH_CHECK(false, name, ": dtype ", t.scalar_type(), " is not supported (fp16, bf16, fp32)");
+        case at::kDouble: return BA_F64;
+        case at::kByte: return BA_U8;
+        case at::kChar: return BA_I8;
+        case at::kShort: return BA_I16;
+        case at::kInt: return BA_I32;
+        case at::kLong: return BA_I64;
+        default: TORCH_CHECK(false, name, ": dtype ", t.scalar_type(), " is not supported");
     }
     return -1;
 }

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BA_ABI_VERSION 2
+#define BA_ABI_VERSION 3
 
 typedef void *ba_stream_t; /* hipStream_t */
 
@@ -41,7 +41,13 @@ typedef enum ba_status {
     BA_ERR_BAD_METADATA = 5  /* ba_plan_read: the device-side checks rejected segments */
 } ba_status;
 
-typedef enum ba_dtype { BA_F16 = 0, BA_BF16 = 1, BA_F32 = 2 } ba_dtype;
+/* Element types: the set of the reference's AT_DISPATCH_ALL_TYPES_AND2(Half, BFloat16)
+ * (csrc/cuda/spBlkGEMM.cu:1010).  The softmax takes the four floating types
+ * (csrc/cuda/spBlkSoftmax.cu:400), the fused pair and the attention BA_F16 / BA_BF16. */
+typedef enum ba_dtype {
+    BA_F16 = 0, BA_BF16 = 1, BA_F32 = 2, BA_F64 = 3,
+    BA_U8 = 4, BA_I8 = 5, BA_I16 = 6, BA_I32 = 7, BA_I64 = 8
+} ba_dtype;
 
 /* Which half of the metadata the caller supplies
  * (the three cases of csrc/sparseBlockedAttention.cpp:22-44). */
@@ -136,7 +142,9 @@ int ba_plan_read(const void *plan, ba_plan_info *host_info, ba_stream_t stream);
  * the plan's totals, otherwise the kernel writes nothing and records a run
  * error in the plan.  transpose1/transpose2 select the K x M / K x N segment
  * layouts (spBlkGEMM.cu:292-329, 363-400).  dtype: BA_F16, BA_BF16 (MFMA,
- * fp32 accumulate) or BA_F32.
+ * fp32 accumulate), or any other ba_dtype with the reference's generic kernel's
+ * arithmetic (spBlkGEMM.cu:159: the accumulator has the element type; integer
+ * results are exact modulo 2^bits).
  */
 int ba_varlen_gemm(void *plan, const ba_plan_info *info, int64_t nseg, int dtype, const void *A, const void *B, void *out,
                    int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
@@ -144,7 +152,8 @@ int ba_varlen_gemm(void *plan, const ba_plan_info *info, int64_t nseg, int dtype
 
 /*
  * dst row = softmax(scale * src row) for every row of every segment, computed
- * in fp32, one rounding at the store.  Stands in for sparseBlockedSoftmaxLaunch
+ * in fp32 (BA_F64: in double), one rounding at the store.  dtype: BA_F16,
+ * BA_BF16, BA_F32 or BA_F64 (likewise in the backward below).  Stands in for sparseBlockedSoftmaxLaunch
  * (csrc/sparseBlockedAttention.h:20, csrc/cuda/spBlkSoftmax.cu:375-416);
  * scale = 1.0f reproduces it.  No column limit.  src == dst is allowed.
  */

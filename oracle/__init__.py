@@ -14,6 +14,12 @@ Two independent statements of the same results live here:
 them with closed forms (uniform scores give column means, one-hot values return
 the probabilities, a dominant key returns its value row) and a brute-force loop.
 
+``varlen_gemm_typed`` / ``blocked_softmax_f64`` restate the same operators for the
+other element types of the reference's dispatch (fp64; uint8, int8, int16, int32,
+int64 with the accumulator in the element type); tests/test_oracle_values.py pins
+them with the arange closed form reduced modulo 2^bits, numpy's wrapping integer
+matmul, numpy / scipy in float64 and torch.autograd in float64.
+
 Both follow the semantics of the reference at
 csrc/sparseBlockedAttention.cpp:11-50, 81-101, csrc/cuda/spBlkGEMM.cu:133-150,
 292-329, 363-400, 985-1008 and csrc/cuda/spBlkSoftmax.cu:95-136, 375-398.
@@ -129,6 +135,56 @@ def varlen_gemm(A, Bm, M, N, K, transpose1=False, transpose2=False, f64acc=False
     fn(pA, pB, out.ctypes.data_as(_F32P), c(H), c(int(a1[-1])), c(int(a2[-1])), c(int(ao[-1])),
        c(M.shape[0]), a1.ctypes.data_as(_I64P), a2.ctypes.data_as(_I64P), ao.ctypes.data_as(_I64P),
        pM, pN, pK, ctypes.c_int(int(transpose1)), ctypes.c_int(int(transpose2)))
+    return out
+
+
+_INT_BITS = {"uint8": (8, 0), "int8": (8, 1), "int16": (16, 1), "int32": (32, 1), "int64": (64, 1)}
+
+
+def varlen_gemm_typed(A, Bm, M, N, K, transpose1=False, transpose2=False):
+    """The generic kernel for the element type of A: float64 (accumulated in double) or one of the integer
+    types (exact modulo 2^bits).  A: [H, Dm1], Bm: [H, Dm2] numpy arrays of one dtype -> [H, Dout], same dtype."""
+    A = np.ascontiguousarray(A); Bm = np.ascontiguousarray(Bm)
+    assert A.dtype == Bm.dtype
+    M, pM = _i64(M); N, pN = _i64(N); K, pK = _i64(K)
+    a1, a2, ao = lists_to_accum(M, N, K)
+    H = A.shape[0]
+    assert A.shape[1] == a1[-1] and Bm.shape[1] == a2[-1] and Bm.shape[0] == H
+    c = ctypes.c_int64
+    meta = (c(H), c(int(a1[-1])), c(int(a2[-1])), c(int(ao[-1])), c(M.shape[0]), a1.ctypes.data_as(_I64P),
+            a2.ctypes.data_as(_I64P), ao.ctypes.data_as(_I64P), pM, pN, pK, ctypes.c_int(int(transpose1)),
+            ctypes.c_int(int(transpose2)))
+    if A.dtype == np.float64:
+        out = np.empty((H, int(ao[-1])), np.float64)
+        P = ctypes.POINTER(ctypes.c_double)
+        lib().oracle_varlen_gemm_f64(A.ctypes.data_as(P), Bm.ctypes.data_as(P), out.ctypes.data_as(P), *meta)
+        return out
+    bits, signed = _INT_BITS[A.dtype.name]
+    a64 = np.ascontiguousarray(A.astype(np.int64)); b64 = np.ascontiguousarray(Bm.astype(np.int64))
+    out = np.empty((H, int(ao[-1])), np.int64)
+    lib().oracle_varlen_gemm_i64(a64.ctypes.data_as(_I64P), b64.ctypes.data_as(_I64P), out.ctypes.data_as(_I64P), *meta,
+                                 ctypes.c_int(bits), ctypes.c_int(signed))
+    return out.astype(A.dtype)          # values already lie in the type's range
+
+
+def blocked_softmax_f64(src, rows, cols, scale=1.0, dy=None):
+    """Row softmax of float64 [H, D] (dy given: its backward, src then being the forward output)."""
+    src = np.ascontiguousarray(src, np.float64)
+    rows, pR = _i64(rows); cols, pC = _i64(cols)
+    accum = softmax_accum(rows, cols)
+    H = src.shape[0]
+    assert src.shape[1] == accum[-1]
+    out = np.empty_like(src)
+    P = ctypes.POINTER(ctypes.c_double)
+    c = ctypes.c_int64
+    if dy is None:
+        lib().oracle_blocked_softmax_f64(src.ctypes.data_as(P), out.ctypes.data_as(P), c(H), c(int(accum[-1])),
+                                         c(rows.shape[0]), accum.ctypes.data_as(_I64P), pR, pC, ctypes.c_double(scale))
+    else:
+        dy = np.ascontiguousarray(dy, np.float64)
+        lib().oracle_blocked_softmax_backward_f64(src.ctypes.data_as(P), dy.ctypes.data_as(P), out.ctypes.data_as(P), c(H),
+                                                  c(int(accum[-1])), c(rows.shape[0]), accum.ctypes.data_as(_I64P), pR, pC,
+                                                  ctypes.c_double(scale))
     return out
 
 

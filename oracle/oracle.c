@@ -227,6 +227,69 @@ ORACLE_API void oracle_varlen_gemm_f64acc(const float *A, const float *Bm, float
         }
 }
 
+/*
+ * The same kernel for T = double (csrc/cuda/spBlkGEMM.cu:1010 instantiates it for every element type;
+ * :159 accumulates in T).
+ */
+ORACLE_API void oracle_varlen_gemm_f64(const double *A, const double *Bm, double *out, int64_t H,
+                                       int64_t Dm1, int64_t Dm2, int64_t Dout, int64_t nseg,
+                                       const int64_t *accum1, const int64_t *accum2, const int64_t *accumOut,
+                                       const int64_t *M, const int64_t *N, const int64_t *K,
+                                       int transpose1, int transpose2) {
+    for (int64_t h = 0; h < H; ++h)
+        for (int64_t g = 0; g < nseg; ++g) {
+            const double *a = A + h * Dm1 + accum1[g];
+            const double *b = Bm + h * Dm2 + accum2[g];
+            double *o = out + h * Dout + accumOut[g];
+            const int64_t m = M[g], n = N[g], k = K[g];
+            for (int64_t r = 0; r < m; ++r)
+                for (int64_t c = 0; c < n; ++c) {
+                    double acc = 0.0;
+                    for (int64_t t = 0; t < k; ++t) {
+                        double av = transpose1 ? a[t * m + r] : a[r * k + t];
+                        double bv = transpose2 ? b[t * n + c] : b[c * k + t];
+                        acc += av * bv;
+                    }
+                    o[r * n + c] = acc;
+                }
+        }
+}
+
+/*
+ * ... and for the integer element types (uint8, int8, int16, int32, int64).  The accumulator has the
+ * element type (:159), so every partial sum is reduced modulo 2^bits; since that reduction commutes with
+ * sums and products, the result is the exact sum of products reduced once at the end.  Operands and
+ * results travel as int64 holding values of the element type; bits in {8, 16, 32, 64}, is_signed says
+ * how the low bits of the result are read.
+ */
+ORACLE_API void oracle_varlen_gemm_i64(const int64_t *A, const int64_t *Bm, int64_t *out, int64_t H,
+                                       int64_t Dm1, int64_t Dm2, int64_t Dout, int64_t nseg,
+                                       const int64_t *accum1, const int64_t *accum2, const int64_t *accumOut,
+                                       const int64_t *M, const int64_t *N, const int64_t *K,
+                                       int transpose1, int transpose2, int bits, int is_signed) {
+    for (int64_t h = 0; h < H; ++h)
+        for (int64_t g = 0; g < nseg; ++g) {
+            const int64_t *a = A + h * Dm1 + accum1[g];
+            const int64_t *b = Bm + h * Dm2 + accum2[g];
+            int64_t *o = out + h * Dout + accumOut[g];
+            const int64_t m = M[g], n = N[g], k = K[g];
+            for (int64_t r = 0; r < m; ++r)
+                for (int64_t c = 0; c < n; ++c) {
+                    uint64_t acc = 0;                     /* wraps modulo 2^64, a multiple of 2^bits */
+                    for (int64_t t = 0; t < k; ++t) {
+                        uint64_t av = (uint64_t)(transpose1 ? a[t * m + r] : a[r * k + t]);
+                        uint64_t bv = (uint64_t)(transpose2 ? b[t * n + c] : b[c * k + t]);
+                        acc += av * bv;
+                    }
+                    if (bits < 64) {
+                        acc &= (((uint64_t)1) << bits) - 1;
+                        if (is_signed && (acc >> (bits - 1))) acc |= ~((((uint64_t)1) << bits) - 1);
+                    }
+                    o[r * n + c] = (int64_t)acc;
+                }
+        }
+}
+
 /* ------------------------------------------------------------------ softmax */
 
 /*
@@ -254,6 +317,48 @@ ORACLE_API void oracle_blocked_softmax_f32(const float *src, float *out, int64_t
                 for (int64_t c = 0; c < nc; ++c) sum += exp((double)x[c] * (double)scale - mx);
                 for (int64_t c = 0; c < nc; ++c)
                     y[c] = (float)(exp((double)x[c] * (double)scale - mx) / sum);
+            }
+        }
+}
+
+/*
+ * The same for T = double (csrc/cuda/spBlkSoftmax.cu:400 instantiates the kernels for double as well),
+ * evaluated in long double and rounded to double once; and its backward.
+ */
+ORACLE_API void oracle_blocked_softmax_f64(const double *src, double *out, int64_t H, int64_t Dsrc, int64_t nseg,
+                                           const int64_t *accum, const int64_t *rows, const int64_t *cols,
+                                           double scale) {
+    for (int64_t h = 0; h < H; ++h)
+        for (int64_t g = 0; g < nseg; ++g) {
+            const int64_t nc = cols[g];
+            for (int64_t r = 0; r < rows[g]; ++r) {
+                const double *x = src + h * Dsrc + accum[g] + r * nc;
+                double *y = out + h * Dsrc + accum[g] + r * nc;
+                long double mx = -INFINITY;
+                for (int64_t c = 0; c < nc; ++c) {
+                    long double v = (long double)x[c] * (long double)scale;
+                    if (v > mx) mx = v;
+                }
+                long double sum = 0.0L;
+                for (int64_t c = 0; c < nc; ++c) sum += expl((long double)x[c] * (long double)scale - mx);
+                for (int64_t c = 0; c < nc; ++c)
+                    y[c] = (double)(expl((long double)x[c] * (long double)scale - mx) / sum);
+            }
+        }
+}
+
+ORACLE_API void oracle_blocked_softmax_backward_f64(const double *y, const double *dy, double *dx, int64_t H,
+                                                    int64_t Dsrc, int64_t nseg, const int64_t *accum,
+                                                    const int64_t *rows, const int64_t *cols, double scale) {
+    for (int64_t h = 0; h < H; ++h)
+        for (int64_t g = 0; g < nseg; ++g) {
+            const int64_t nc = cols[g];
+            for (int64_t r = 0; r < rows[g]; ++r) {
+                const int64_t base = h * Dsrc + accum[g] + r * nc;
+                long double dot = 0.0L;
+                for (int64_t c = 0; c < nc; ++c) dot += (long double)y[base + c] * (long double)dy[base + c];
+                for (int64_t c = 0; c < nc; ++c)
+                    dx[base + c] = (double)((long double)scale * ((long double)dy[base + c] - dot) * (long double)y[base + c]);
             }
         }
 }

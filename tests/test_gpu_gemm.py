@@ -137,7 +137,7 @@ def test_many_tiny_segments_are_packed(dev):
 
 def test_unsupported_dtype_and_empty_calls(dev):
     plan = make_plan(dev, [4], [4], [8])
-    x = torch.zeros((1, 32), dtype=torch.float64, device=dev)
+    x = torch.zeros((1, 32), dtype=torch.complex64, device=dev)     # not one of the reference's dispatch types
     with pytest.raises(capi.BlockedAttentionError, match="unsupported dtype"):
         capi.varlen_gemm(plan, x, x, x, 1, 32, 32, 16)
     e = torch.empty((0, 32), dtype=torch.float16, device=dev)

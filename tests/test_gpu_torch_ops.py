@@ -86,7 +86,7 @@ def test_errors_are_runtime_errors(dev):
     with pytest.raises(RuntimeError, match="rejected"):
         blockedAttention.blockGEMM(A, A, MList=dl([-4], dev), NList=N, KList=K)
     with pytest.raises(RuntimeError, match="not supported"):
-        blockedAttention.blockGEMM(A.double(), A.double(), MList=M, NList=N, KList=K)
+        blockedAttention.blockGEMM(A.to(torch.complex64), A.to(torch.complex64), MList=M, NList=N, KList=K)
     empty = blockedAttention.blockGEMM(A[:, :0], A[:, :0], MList=dl([], dev), NList=dl([], dev), KList=dl([], dev))
     assert empty.shape == (1, 0)
 

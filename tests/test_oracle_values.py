@@ -202,3 +202,73 @@ def test_attention_two_statements_agree():
     a = oracle.attention(Q, Km, V, M, N, K, 0.3)
     b = oracle.per_segment_torch_attention(torch.from_numpy(Q), torch.from_numpy(Km), torch.from_numpy(V), M, N, K, 0.3)
     assert np.allclose(a, b.numpy(), rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- the other element types
+@pytest.mark.parametrize("dtype", ["int64", "int32", "int16", "int8", "uint8"])
+def test_integer_gemm_closed_form_11_13_5(dtype):
+    # the reference's arange case again, in the integer types; for the narrow ones the closed form is reduced
+    # modulo 2^bits (the accumulator has the element type, csrc/cuda/spBlkGEMM.cu:159)
+    A = np.arange(55).astype(dtype)[None]
+    B = np.arange(65).astype(dtype)[None]
+    out = oracle.varlen_gemm_typed(A, B, [11], [13], [5])
+    exact = np.array([[sum((5 * r + t) * (5 * c + t) for t in range(5)) for c in range(13)] for r in range(11)])
+    assert out.dtype == np.dtype(dtype)
+    assert np.array_equal(out.reshape(11, 13), exact.astype(np.int64).astype(dtype))      # astype wraps
+    if dtype in ("int64", "int32"):
+        assert np.array_equal(out.reshape(11, 13).astype(np.int64), exact)                # no wrap at these sizes
+
+
+@pytest.mark.parametrize("dtype", ["int64", "int32", "int16", "int8", "uint8"])
+@pytest.mark.parametrize("t1,t2", [(False, False), (True, True)])
+def test_integer_gemm_wraps_like_numpy(dtype, t1, t2):
+    # numpy's integer matmul keeps the element type and wraps: an independent statement of the same arithmetic
+    rng = np.random.default_rng(5)
+    info = np.iinfo(dtype)
+    M, N, K = np.array([5, 8, 1]), np.array([4, 3, 6]), np.array([70, 2, 90])
+    H = 2
+    A = rng.integers(info.min, info.max, (H, int((M * K).sum())), dtype=dtype, endpoint=True)
+    Bm = rng.integers(info.min, info.max, (H, int((N * K).sum())), dtype=dtype, endpoint=True)
+    out = oracle.varlen_gemm_typed(A, Bm, M, N, K, transpose1=t1, transpose2=t2)
+    o1 = o2 = oo = 0
+    for m, n, k in zip(M, N, K):
+        a = A[:, o1:o1 + m * k].reshape(H, k, m).transpose(0, 2, 1) if t1 else A[:, o1:o1 + m * k].reshape(H, m, k)
+        b = Bm[:, o2:o2 + n * k].reshape(H, k, n).transpose(0, 2, 1) if t2 else Bm[:, o2:o2 + n * k].reshape(H, n, k)
+        with np.errstate(over="ignore"):
+            ref = np.matmul(a, b.transpose(0, 2, 1))
+        assert ref.dtype == np.dtype(dtype)
+        assert np.array_equal(out[:, oo:oo + m * n].reshape(H, m, n), ref)
+        o1 += m * k; o2 += n * k; oo += m * n
+
+
+def test_f64_gemm_matches_numpy_and_the_closed_form():
+    A = np.arange(55, dtype=np.float64)[None]; B = np.arange(65, dtype=np.float64)[None]
+    exact = np.array([[sum((5 * r + t) * (5 * c + t) for t in range(5)) for c in range(13)] for r in range(11)])
+    assert np.array_equal(oracle.varlen_gemm_typed(A, B, [11], [13], [5]).reshape(11, 13), exact.astype(np.float64))
+    rng = np.random.default_rng(6)
+    M, N, K = np.array([5, 8, 1]), np.array([4, 3, 6]), np.array([70, 2, 90])
+    A = rng.standard_normal((2, int((M * K).sum()))); Bm = rng.standard_normal((2, int((N * K).sum())))
+    out = oracle.varlen_gemm_typed(A, Bm, M, N, K, transpose2=True)
+    o1 = o2 = oo = 0
+    for m, n, k in zip(M, N, K):
+        a = A[:, o1:o1 + m * k].reshape(2, m, k); b = Bm[:, o2:o2 + n * k].reshape(2, k, n)
+        np.testing.assert_allclose(out[:, oo:oo + m * n].reshape(2, m, n), np.matmul(a, b), rtol=1e-13, atol=1e-13)
+        o1 += m * k; o2 += n * k; oo += m * n
+
+
+def test_f64_softmax_matches_scipy_and_autograd():
+    rng = np.random.default_rng(7)
+    rows, cols = np.array([3, 5, 1]), np.array([7, 300, 2])
+    x = rng.standard_normal((2, int((rows * cols).sum()))) * 4
+    y = oracle.blocked_softmax_f64(x, rows, cols, scale=0.7)
+    dy = rng.standard_normal(x.shape)
+    dx = oracle.blocked_softmax_f64(y, rows, cols, scale=0.7, dy=dy)
+    o = 0
+    for r, c in zip(rows, cols):
+        seg = x[:, o:o + r * c].reshape(2, r, c)
+        np.testing.assert_allclose(y[:, o:o + r * c].reshape(2, r, c), scipy.special.softmax(0.7 * seg, axis=-1),
+                                   rtol=1e-14, atol=1e-16)
+        t = torch.tensor(seg, dtype=torch.float64, requires_grad=True)
+        torch.softmax(0.7 * t, dim=-1).backward(torch.tensor(dy[:, o:o + r * c].reshape(2, r, c)))
+        np.testing.assert_allclose(dx[:, o:o + r * c].reshape(2, r, c), t.grad.numpy(), rtol=1e-12, atol=1e-14)
+        o += r * c
