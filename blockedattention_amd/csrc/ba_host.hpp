@@ -53,6 +53,8 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
 // BA_ERR_UNSUPPORTED when the plan summary is missing or does not fit; the caller then takes launch_tiles.
 int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                      hipStream_t stream);
+// fp16 / bf16 in any layout and alignment (gemm_any16.hip: both operands staged through LDS, MFMA)
+int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 // fp32, fp64 and the integer types (gemm_generic.hip); dtype: ba_dtype
 int launch_gemm_generic(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,

@@ -63,7 +63,7 @@ enum PrefixKind {
     kPfxRows = 9,   // softmax: M rows
     kPfxPack = 10,  // 1 for the first segment of a pack of tiny segments, else 0
     kPfxSlow = 11,  // ceil(M/16) for segments the 16-byte operand loads cannot serve
-    kPfxAtt64 = 12,   // one-pass attention, GEMM plans: ceil(M/64) for segments with rows and a head dimension
+    kPfxAtt64 = 12,   // GEMM plans: ceil(M/64) for every segment with rows (one-pass attention, any-layout GEMM)
     kPfxAtt128 = 13,  // the same in row blocks of 128
     kNumPrefix = 14
 };

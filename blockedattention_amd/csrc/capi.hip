@@ -149,6 +149,11 @@ __attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_p
     if (transpose2) args.flags |= kFlagTranspose2;
     args.flags |= mfma_flag(args);
     if (dtype != BA_F16 && dtype != BA_BF16) return launch_gemm_generic(dtype, args, nseg, info, (hipStream_t)stream);
+    // Transposed layouts and unaligned operands, or a batch most of whose segments break the 16-byte operand
+    // alignment (reduction lengths that are not multiples of 8, as in the backward products): the kernel that
+    // stages both operands through LDS.  Everything else: the strip, tile and segment kernels.
+    if (!(args.flags & kFlagMfmaOk) || (info && info->slow_items > 0 && 32 * info->slow_items > info->total_rows))
+        return launch_gemm_any16(dtype, args, nseg, info, (hipStream_t)stream);
     return launch_strips(dtype, 0, args, nseg, info, (hipStream_t)stream);
 }
 

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         v32[kPfxRows] = ni >= 1 ? mi : 0;
         v32[kPfxPack] = pack > 0 ? 1 : 0;
         v32[kPfxSlow] = aligned ? 0 : strips;
-        const bool att_rows = mi >= 1 && ki >= 1;              // the attention kernel works on these, whatever N is
+        const bool att_rows = mi >= 1;                         // row blocks of every segment with rows, whatever N and K are
         v32[kPfxAtt64] = att_rows ? (mi + kAttBlockRows - 1) / kAttBlockRows : 0;
         v32[kPfxAtt128] = att_rows ? (mi + 2 * kAttBlockRows - 1) / (2 * kAttBlockRows) : 0;
         if (a.kind == 1) {

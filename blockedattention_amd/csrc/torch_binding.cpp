@@ -84,7 +84,7 @@ struct Schedule;
 // use and shared by every copy of the schedule, so that they live and die with its cache entry.
 struct Derived {
     std::mutex mu;
-    std::shared_ptr<Schedule> padded, grad1, grad2;
+    std::shared_ptr<Schedule> grad1, grad2;
 };
 
 struct Schedule {
@@ -176,14 +176,14 @@ std::vector<int64_t> schedule_cache_stats() {
 
 // The three metadata cases of the reference (cpp:17-44), resolved on the device.
 Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor &a2, const OptTensor &aO,
-                       const OptTensor &M, const OptTensor &N, const OptTensor &K) {
+                       const OptTensor &M, const OptTensor &N, const OptTensor &K, bool use_cache = true) {
     const bool have_accum = a1.has_value() && a2.has_value() && aO.has_value();
     const bool have_lists = M.has_value() && N.has_value() && K.has_value();
     TORCH_CHECK(have_accum || have_lists,
                 "sparseBlockedGEMM needs either (mat1Accum, mat2Accum, outAccum) or (MList, NList, KList)");
     Schedule s;
     const ScheduleKey key = make_key(0, like, {&a1, &a2, &aO, &M, &N, &K});
-    if (cache_lookup(key, s)) return s;
+    if (use_cache && cache_lookup(key, s)) return s;
     s.derived = std::make_shared<Derived>();
     int64_t nseg;
     int mode;
@@ -222,7 +222,7 @@ Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor 
     TORCH_CHECK(st != BA_ERR_BAD_METADATA, "segment metadata rejected: ", s.info.bad_segments,
                 " segment(s) have negative, oversized or inconsistent shapes / prefix sums");
     check_status(st, "ba_plan_read");
-    cache_store(key, s);
+    if (use_cache) cache_store(key, s);
     return s;
 }
 
@@ -273,56 +273,19 @@ Tensor gemm_launch(const Tensor &mat1, const Tensor &mat2, Schedule &s, bool t1,
     return out;
 }
 
-Tensor ceil8(const Tensor &t) { return at::mul(at::floor_divide(at::add(t, 7), 8), 8); }
-
-// One operand of a repacked product: which operand of the source schedule it is, whether its dimensions
-// swap, and whether it is stored column-major with respect to the (swapped) dimensions.
-struct Repack {
-    const Tensor &data;
-    int which;
-    bool swap, column_major;
-};
-
-// out_g = L1_g L2_g^T on the MFMA path for 16-bit operands in any layout and with any reduction length:
-// both operands are first repacked (csrc/repack.hip) into zero-padded row-major rows of a multiple of 8
-// elements, under the schedule `dst` whose lists are (rows of L1, rows of L2, padded reduction length).
-Tensor gemm_repacked(const Schedule &src, Schedule &dst, const Repack &p1, const Repack &p2) {
-    const Tensor &like = p1.data;
-    const int64_t H = leading(p1.data);
-    TORCH_CHECK(leading(p2.data) == H, "the operands disagree on the number of heads");
-    const int dt = dtype_code(like, "sparseBlockedGEMM");
-    void *stream = current_stream(like);
-    Tensor x = at::empty({H, dst.info.Dm1}, like.options()), y = at::empty({H, dst.info.Dm2}, like.options());
-    check_status(ba_repack_operand(src.plan.data_ptr(), p1.which, p1.swap, p1.column_major, dst.plan.data_ptr(), 0,
-                                   &dst.info, src.info.nseg, dt, p1.data.data_ptr(), x.data_ptr(), H, p1.data.size(-1),
-                                   dst.info.Dm1, stream),
-                 "ba_repack_operand");
-    check_status(ba_repack_operand(src.plan.data_ptr(), p2.which, p2.swap, p2.column_major, dst.plan.data_ptr(), 1,
-                                   &dst.info, src.info.nseg, dt, p2.data.data_ptr(), y.data_ptr(), H, p2.data.size(-1),
-                                   dst.info.Dm2, stream),
-                 "ba_repack_operand");
-    Tensor out = at::empty({H, dst.info.Dout}, like.options());
-    check_status(ba_varlen_gemm(dst.plan.data_ptr(), &dst.info, dst.info.nseg, dt, x.data_ptr(), y.data_ptr(), out.data_ptr(),
-                                H, dst.info.Dm1, dst.info.Dm2, dst.info.Dout, 0, 0, stream),
-                 "ba_varlen_gemm");
-    return out;
-}
-
-// The derived schedule `slot` of s over the lists (rows, cols, ceil8(reduce)), made once.
+// The schedule of one of the two backward products of s (permuted metadata, given in both forms), made once and
+// kept with s: it lives and dies with the forward schedule and takes no slot of the cache.
 Schedule &derived_schedule(const Schedule &s, std::shared_ptr<Schedule> Derived::*slot, const Tensor &like,
-                           const Tensor &rows, const Tensor &cols, const Tensor &reduce) {
+                           const Tensor &a1, const Tensor &a2, const Tensor &aO, const Tensor &rows, const Tensor &cols,
+                           const Tensor &reduce) {
     TORCH_CHECK(s.derived, "internal: schedule without a holder for derived schedules");
     std::lock_guard<std::mutex> lock(s.derived->mu);
     std::shared_ptr<Schedule> &p = (*s.derived).*slot;
-    if (!p) {
-        const OptTensor none;
-        p = std::make_shared<Schedule>(schedule_gemm(like, none, none, none, OptTensor(rows), OptTensor(cols),
-                                                     OptTensor(ceil8(reduce))));
-    }
+    if (!p)
+        p = std::make_shared<Schedule>(schedule_gemm(like, OptTensor(a1), OptTensor(a2), OptTensor(aO), OptTensor(rows),
+                                                     OptTensor(cols), OptTensor(reduce), /*use_cache=*/false));
     return *p;
 }
-
-bool is_16bit(const Tensor &t) { return t.scalar_type() == at::kHalf || t.scalar_type() == at::kBFloat16; }
 
 class SparseBlockedGEMM : public torch::autograd::Function<SparseBlockedGEMM> {
 public:
@@ -335,12 +298,6 @@ public:
         ctx->save_for_backward({mat1, mat2, s.accum1, s.accum2, s.accumOut, s.M, s.N, s.K});
         ctx->saved_data["transpose1"] = t1;
         ctx->saved_data["transpose2"] = t2;
-        if (is_16bit(mat1) && mat1.scalar_type() == mat2.scalar_type() && (t1 || t2 || s.info.slow_items > 0) &&
-            mat1.dim() >= 1 && mat2.dim() >= 1 && mat1.size(-1) == s.info.Dm1 && mat2.size(-1) == s.info.Dm2) {
-            // transposed layouts or reduction lengths that are not multiples of 8: repack, then the MFMA path
-            Schedule &padded = derived_schedule(s, &Derived::padded, mat1, s.M, s.N, s.K);
-            return {gemm_repacked(s, padded, Repack{mat1, 0, false, t1}, Repack{mat2, 1, false, t2})};
-        }
         return {gemm_launch(mat1, mat2, s, t1, t2)};
     }
 
@@ -355,19 +312,13 @@ public:
         const Tensor &a1 = saved[2], &a2 = saved[3], &aO = saved[4], &M = saved[5], &N = saved[6], &K = saved[7];
         const bool t1 = ctx->saved_data["transpose1"].toBool(), t2 = ctx->saved_data["transpose2"].toBool();
         Tensor g1, g2;
-        if (is_16bit(grad)) {
-            // dA = dS B reduces over N, dB = dS^T A over M: repack (transpose + pad), then the MFMA path
-            Schedule fwd = schedule_gemm(grad, a1, a2, aO, M, N, K);
-            Schedule &sa = derived_schedule(fwd, &Derived::grad1, grad, M, K, N);
-            g1 = gemm_repacked(fwd, sa, Repack{grad, 2, false, false}, Repack{mat2, 1, true, !t2});
-            Schedule &sb = derived_schedule(fwd, &Derived::grad2, grad, N, K, M);
-            g2 = gemm_repacked(fwd, sb, Repack{grad, 2, true, true}, Repack{mat1, 0, true, !t1});
-        } else {
-            Schedule s1 = schedule_gemm(grad, aO, a2, a1, M, K, N);
-            g1 = gemm_launch(grad, mat2, s1, false, !t2);
-            Schedule s2 = schedule_gemm(grad, aO, a1, a2, N, K, M);
-            g2 = gemm_launch(grad, mat1, s2, true, !t1);
-        }
+        // dS and the saved operands are read as they lie: the products whose reduction runs over N or M take the
+        // kernels for any layout and reduction length (two launches, like the reference)
+        Schedule fwd = schedule_gemm(grad, a1, a2, aO, M, N, K);          // the forward's, from the cache
+        Schedule &s1 = derived_schedule(fwd, &Derived::grad1, grad, aO, a2, a1, M, K, N);
+        g1 = gemm_launch(grad, mat2, s1, false, !t2);
+        Schedule &s2 = derived_schedule(fwd, &Derived::grad2, grad, aO, a1, a2, N, K, M);
+        g2 = gemm_launch(grad, mat1, s2, true, !t1);
         return {g1.view_as(saved[0]), g2.view_as(saved[1]), Tensor(), Tensor(), Tensor(), Tensor(), Tensor(),
                 Tensor(), Tensor(), Tensor()};
     }

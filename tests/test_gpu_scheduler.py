@@ -151,7 +151,7 @@ def test_empty_batch(dev):
 
 def test_row_block_prefixes_of_the_attention_work_list(dev):
     # Behind the work lists the plan keeps, for blocks of 64 and of 128 rows, how many row blocks the segments
-    # before each segment have (segments without rows or without a head dimension have none); entry nseg = total.
+    # before each segment have (every segment with rows counts, whatever its N and K); entry nseg = total.
     rng = np.random.default_rng(11)
     for nseg in (1, 63, 300, 2500):
         M = rng.integers(0, 700, nseg); N = rng.integers(0, 40, nseg); K = rng.choice([0, 8, 64], nseg)
@@ -159,7 +159,7 @@ def test_row_block_prefixes_of_the_attention_work_list(dev):
         cap = (nseg + 4) & ~3
         words = plan.buf.cpu().numpy()[256 + 6 * 48 * cap:].view(np.int32)
         for which, rows in ((0, 64), (1, 128)):
-            blocks = np.where((M >= 1) & (K >= 1), (M + rows - 1) // rows, 0)
+            blocks = np.where(M >= 1, (M + rows - 1) // rows, 0)
             want = np.concatenate([[0], np.cumsum(blocks)]).astype(np.int32)
             got = words[which * (cap + 4): which * (cap + 4) + nseg + 1]
             assert np.array_equal(got, want), (nseg, rows)
