@@ -116,6 +116,9 @@ class Case:
                        c._ptr(self.att), *dims, f32(w.scale), st)
         self._a_gemm = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.scores),
                         *dims, i32(0), i32(0), st)
+        # the same call with both operands read as K x M / K x N (any-layout kernel; the buffers hold as many elements)
+        self._a_gemm_t = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.A), c._ptr(self.B), c._ptr(self.scores),
+                          *dims, i32(1), i32(1), st)
         self._a_soft = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.scores), c._ptr(self.out), i64(w.heads),
                         i64(w.Dout), f32(w.scale), st)
         for st_code, what in ((lib.ba_plan_gemm(*self._a_sched), "ba_plan_gemm"),
@@ -133,6 +136,9 @@ class Case:
 
     def gemm(self):
         self._lib.ba_varlen_gemm(*self._a_gemm)
+
+    def gemm_transposed(self):
+        self._lib.ba_varlen_gemm(*self._a_gemm_t)
 
     def softmax(self):
         self._lib.ba_blocked_softmax(*self._a_soft)
@@ -276,7 +282,29 @@ class Case:
             fig["gemm_only_us"] = round(self.event_us(self.gemm, steps, warmup), 3)
             fig["softmax_only_us"] = round(self.event_us(self.softmax, steps, warmup), 3)
             fig["unfused_pair_us"] = round(self.event_us(self.unfused, steps, warmup), 3)
+            fig["gemm_transposed_us"] = round(self.event_us(self.gemm_transposed, steps, warmup), 3)
+            fig.update(self.backward_figures(max(10, steps // 5), 5))
         return fig
+
+    def backward_figures(self, steps, warmup):
+        """GEMM then softmax through the torch operators, and their backward (two softmax-backward-sized passes and
+        the two products dA = dS B, dB = dS^T A, read as they lie)."""
+        torch, w = self.torch, self.w
+        try:
+            import blockAttention
+        except ImportError as e:
+            return {"backward_us": f"extension not built: {e}"}
+        A = self.A.detach().clone().requires_grad_(True); B = self.B.detach().clone().requires_grad_(True)
+        dY = torch.randn(w.heads, w.Dout, device=self.dev, dtype=w.dtype)
+        def fwd():
+            S = blockAttention.sparseBlockedGEMM(A, B, None, None, None, self.M, self.N, self.K, False, False)
+            return blockAttention.sparseBlockedSoftmax(S, self.M, self.N, None)
+        def both():
+            A.grad = None; B.grad = None
+            fwd().backward(dY)
+        f_us = self.event_us(fwd, steps, warmup); b_us = self.event_us(both, steps, warmup)
+        return {"op_forward_us": round(f_us, 3), "op_backward_us": round(b_us - f_us, 3),
+                "backward_over_forward": round((b_us - f_us) / f_us, 2)}
 
 
 def cpu_baseline(case, seconds):
