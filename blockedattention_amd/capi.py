@@ -17,9 +17,11 @@ META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
 
 SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
+    "ba_plan_read_into", "ba_plan_gemm_notify", "ba_plan_softmax_notify", "ba_plan_wait",
     "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax", "ba_repack_operand",
     "ba_varlen_attention", "ba_gemm_softmax_static",
 )
+MAILBOX_BYTES = 320
 STATIC_MAX_SEGMENTS = 4096   # BA_STATIC_MAX_SEGMENTS
 
 
@@ -69,6 +71,15 @@ def load():
     lib.ba_plan_softmax.argtypes = [vp, ctypes.c_size_t, i64, vp, vp, vp, i32, vp]
     lib.ba_plan_read.restype = i32
     lib.ba_plan_read.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
+    u32 = ctypes.c_uint32
+    lib.ba_plan_read_into.restype = i32
+    lib.ba_plan_read_into.argtypes = [vp, ctypes.POINTER(PlanInfo), vp, vp]
+    lib.ba_plan_gemm_notify.restype = i32
+    lib.ba_plan_gemm_notify.argtypes = [vp, ctypes.c_size_t, i64, i32, vp, vp, vp, vp, vp, vp, vp, u32, vp]
+    lib.ba_plan_softmax_notify.restype = i32
+    lib.ba_plan_softmax_notify.argtypes = [vp, ctypes.c_size_t, i64, vp, vp, vp, i32, vp, u32, vp]
+    lib.ba_plan_wait.restype = i32
+    lib.ba_plan_wait.argtypes = [vp, u32, ctypes.POINTER(PlanInfo), i64]
     lib.ba_varlen_gemm.restype = i32
     lib.ba_varlen_gemm.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]
     lib.ba_blocked_softmax.restype = i32
@@ -139,16 +150,37 @@ class Plan:
         self.info = info
         return info
 
+    def read_into(self, staging, raise_on_bad=True):
+        """As read(), the summary travelling through `staging` (a pinned CPU tensor of at least 256 bytes)."""
+        info = PlanInfo()
+        st = load().ba_plan_read_into(self.ptr, ctypes.byref(info), ctypes.c_void_p(staging.data_ptr()), _stream())
+        if st != 0 and (raise_on_bad or st != 5):
+            check(st, "ba_plan_read_into")
+        self.info = info
+        return info
+
+    def wait(self, mailbox, ticket, timeout_us=10_000_000, raise_on_bad=True):
+        """The summary a *_notify scheduler call wrote into `mailbox` (pinned CPU tensor): spins on the host, no
+        copy and no stream synchronisation."""
+        info = PlanInfo()
+        st = load().ba_plan_wait(ctypes.c_void_p(mailbox.data_ptr()), ticket, ctypes.byref(info), timeout_us)
+        if st != 0 and (raise_on_bad or st != 5):
+            check(st, "ba_plan_wait")
+        self.info = info
+        return info
+
     def _hint(self):
         return ctypes.byref(self.info) if self.info is not None else None
 
 
 def plan_gemm(nseg, device, MList=None, NList=None, KList=None, accum1=None, accum2=None, accumOut=None,
-              mode=None, plan=None):
+              mode=None, plan=None, mailbox=None, ticket=0):
     """Run the scheduler.  Tensors passed as None in an *output* role are not written.
 
     ``plan``: an existing Plan of the same segment count to schedule into again (no allocation, e.g.
-    under stream capture); its host summary is dropped, since it describes the previous schedule."""
+    under stream capture); its host summary is dropped, since it describes the previous schedule.
+    ``mailbox`` (pinned CPU tensor of MAILBOX_BYTES) and ``ticket``: the scheduler also hands the summary to the
+    host there; collect it with ``plan.wait(mailbox, ticket)``."""
     have_lists = MList is not None and NList is not None and KList is not None
     have_accum = accum1 is not None and accum2 is not None and accumOut is not None
     if mode is None:
@@ -162,6 +194,12 @@ def plan_gemm(nseg, device, MList=None, NList=None, KList=None, accum1=None, acc
     elif plan.nseg != int(nseg):
         raise BlockedAttentionError(f"the plan was sized for {plan.nseg} segments, not {nseg}")
     plan.info = None
+    if mailbox is not None:
+        st = load().ba_plan_gemm_notify(plan.ptr, plan.bytes, nseg, mode, _ptr(MList), _ptr(NList), _ptr(KList),
+                                        _ptr(accum1), _ptr(accum2), _ptr(accumOut), ctypes.c_void_p(mailbox.data_ptr()),
+                                        ticket, _stream())
+        check(st, "ba_plan_gemm_notify")
+        return plan
     st = load().ba_plan_gemm(plan.ptr, plan.bytes, nseg, mode, _ptr(MList), _ptr(NList), _ptr(KList),
                              _ptr(accum1), _ptr(accum2), _ptr(accumOut), _stream())
     check(st, "ba_plan_gemm")

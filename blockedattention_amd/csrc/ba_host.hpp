@@ -40,7 +40,8 @@ struct RunArgs {
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,
-                    int64_t *K, int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream);
+                    int64_t *K, int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream, void *mailbox = nullptr,
+                    uint32_t ticket = 0);
 
 // mode 0 = GEMM only, 1 = fused GEMM + softmax.  dtype BA_F16 / BA_BF16.
 // info: optional host copy of the plan summary (from ba_plan_read), or nullptr.

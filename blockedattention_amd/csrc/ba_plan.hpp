@@ -67,6 +67,7 @@ enum PrefixKind {
     kPfxAtt128 = 13,  // the same in row blocks of 128
     kNumPrefix = 14
 };
+constexpr int kMailboxTicket = 256;   // byte offset of the ticket word in a scheduler mailbox (behind the header copy)
 constexpr int kAttBlockRows = 64;   // kPfxAtt64 counts blocks of this many rows, kPfxAtt128 of twice as many
 
 // A segment is "aligned" when K % 8 == 0 and its A and B offsets are multiples

@@ -3,6 +3,7 @@
 // except ba_plan_read.
 #include <string.h>
 
+#include <chrono>
 #include <mutex>
 
 #include "ba_host.hpp"
@@ -96,20 +97,8 @@ __attribute__((visibility("default"))) int ba_plan_softmax(void *plan, size_t pl
                            nullptr, accum, (hipStream_t)stream);
 }
 
-__attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_plan_info *info, ba_stream_t stream) {
-    if (!plan || !info) return BA_ERR_INVALID_ARG;
-    // The header lands in pinned host memory (one 256-byte buffer per calling thread, allocated at the thread's
-    // first call and kept for the life of the process): the copy then needs no staging by the runtime.
-    static thread_local PlanHeader *pinned = [] {
-        void *p = nullptr;
-        return hipHostMalloc(&p, sizeof(PlanHeader), hipHostMallocDefault) == hipSuccess ? (PlanHeader *)p : nullptr;
-    }();
-    PlanHeader on_stack;
-    PlanHeader *dst = pinned ? pinned : &on_stack;
-    if (hipMemcpyAsync(dst, plan, sizeof(PlanHeader), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
-        return BA_ERR_LAUNCH;
-    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return BA_ERR_LAUNCH;
-    const PlanHeader h = *dst;
+// host copy of a plan header -> the public summary
+static int info_from_header(const PlanHeader &h, ba_plan_info *info) {
     if (h.magic != kPlanMagic) return BA_ERR_INVALID_ARG;
     memset(info, 0, sizeof(*info));
     info->nseg = h.nseg;
@@ -134,6 +123,66 @@ __attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_pla
     info->att_blocks64 = h.att_blocks64;
     info->att_blocks128 = h.att_blocks128;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
+}
+
+static int read_header_through(const void *plan, ba_plan_info *info, PlanHeader *staging, hipStream_t stream) {
+    if (hipMemcpyAsync(staging, plan, sizeof(PlanHeader), hipMemcpyDeviceToHost, stream) != hipSuccess) return BA_ERR_LAUNCH;
+    if (hipStreamSynchronize(stream) != hipSuccess) return BA_ERR_LAUNCH;
+    const PlanHeader h = *staging;
+    return info_from_header(h, info);
+}
+
+__attribute__((visibility("default"))) int ba_plan_read(const void *plan, ba_plan_info *info, ba_stream_t stream) {
+    if (!plan || !info) return BA_ERR_INVALID_ARG;
+    // The header lands in pinned host memory (one 256-byte buffer per calling thread, allocated at the thread's
+    // first call and kept for the life of the process): the copy then needs no staging by the runtime.
+    static thread_local PlanHeader *pinned = [] {
+        void *p = nullptr;
+        return hipHostMalloc(&p, sizeof(PlanHeader), hipHostMallocDefault) == hipSuccess ? (PlanHeader *)p : nullptr;
+    }();
+    PlanHeader on_stack;
+    return read_header_through(plan, info, pinned ? pinned : &on_stack, (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_plan_read_into(const void *plan, ba_plan_info *info, void *staging,
+                                                             ba_stream_t stream) {
+    if (!plan || !info || !staging || ((uintptr_t)staging & 15)) return BA_ERR_INVALID_ARG;
+    return read_header_through(plan, info, reinterpret_cast<PlanHeader *>(staging), (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_plan_gemm_notify(void *plan, size_t plan_bytes, int64_t nseg, int mode,
+                                                               int64_t *MList, int64_t *NList, int64_t *KList,
+                                                               int64_t *accum1, int64_t *accum2, int64_t *accumOut,
+                                                               void *mailbox, uint32_t ticket, ba_stream_t stream) {
+    if (!mailbox) return BA_ERR_INVALID_ARG;
+    return launch_schedule(plan, plan_bytes, nseg, mode, 0, MList, NList, KList, accum1, accum2, accumOut,
+                           (hipStream_t)stream, mailbox, ticket);
+}
+
+__attribute__((visibility("default"))) int ba_plan_softmax_notify(void *plan, size_t plan_bytes, int64_t nseg,
+                                                                  const int64_t *rowList, const int64_t *colList,
+                                                                  int64_t *accum, int accum_given, void *mailbox,
+                                                                  uint32_t ticket, ba_stream_t stream) {
+    if (!mailbox) return BA_ERR_INVALID_ARG;
+    return launch_schedule(plan, plan_bytes, nseg, accum_given ? BA_META_GIVEN : BA_META_FROM_LISTS, 1,
+                           const_cast<int64_t *>(rowList), const_cast<int64_t *>(colList), nullptr, nullptr,
+                           nullptr, accum, (hipStream_t)stream, mailbox, ticket);
+}
+
+__attribute__((visibility("default"))) int ba_plan_wait(const void *mailbox, uint32_t ticket, ba_plan_info *info,
+                                                        int64_t timeout_us) {
+    if (!mailbox || !info) return BA_ERR_INVALID_ARG;
+    const uint32_t *word = reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(mailbox) + kMailboxTicket);
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint64_t spins = 0;; ++spins) {
+        if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == ticket) break;
+        if ((spins & 1023) == 1023 && timeout_us >= 0 &&
+            std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count() > timeout_us)
+            return BA_ERR_LAUNCH;
+    }
+    PlanHeader h;
+    memcpy(&h, mailbox, sizeof(PlanHeader));
+    return info_from_header(h, info);
 }
 
 __attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_plan_info *info, int64_t nseg,

@@ -25,6 +25,8 @@ struct SchedArgs {
     int kind;   // 0 GEMM plan, 1 softmax plan
     int64_t *M, *N, *K;
     int64_t *a1, *a2, *aO;
+    void *mailbox;      // host memory the GPU can write, or nullptr: receives a copy of the header, then the ticket
+    uint32_t ticket;
 };
 
 // Exclusive scan of NQ quantities over the workgroup.  Wavefront-level DPP
@@ -332,11 +334,20 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->att_blocks128 = base32[kPfxAtt128];
         plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
         plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
+        if (a.mailbox) {
+            // the summary for a host that waits on the ticket instead of copying and synchronising: the header
+            // first, visible system-wide, then the ticket behind it
+            __builtin_memcpy(a.mailbox, h, sizeof(PlanHeader));
+            __threadfence_system();
+            __hip_atomic_store(reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(a.mailbox) + kMailboxTicket), a.ticket,
+                               __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
     }
 }
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,
-                    int64_t *K, int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream) {
+                    int64_t *K, int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream, void *mailbox,
+                    uint32_t ticket) {
     if (!plan || nseg < 0 || nseg > (int64_t(1) << 30)) return BA_ERR_INVALID_ARG;
     if (plan_bytes < plan_bytes_for(nseg) || ((uintptr_t)plan & 15)) return BA_ERR_WORKSPACE;
     if (mode < 0 || mode > 2) return BA_ERR_INVALID_ARG;
@@ -348,7 +359,8 @@ int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int k
     } else if (need_accum && (!aO || (kind == 0 && (!a1 || !a2)))) {
         return BA_ERR_INVALID_ARG;
     }
-    SchedArgs args{plan, nseg, mode, kind, M, N, K, a1, a2, aO};
+    if (mailbox && ((uintptr_t)mailbox & 15)) return BA_ERR_INVALID_ARG;
+    SchedArgs args{plan, nseg, mode, kind, M, N, K, a1, a2, aO, mailbox, ticket};
     if (nseg <= 64) hipLaunchKernelGGL(schedule_kernel<64>, dim3(1), dim3(64), 0, stream, args);
     else if (nseg <= 256) hipLaunchKernelGGL(schedule_kernel<256>, dim3(1), dim3(256), 0, stream, args);
     else if (nseg <= 512) hipLaunchKernelGGL(schedule_kernel<512>, dim3(1), dim3(512), 0, stream, args);

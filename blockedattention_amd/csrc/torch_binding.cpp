@@ -174,6 +174,22 @@ std::vector<int64_t> schedule_cache_stats() {
     return {c.hits, c.misses, (int64_t)c.entries.size(), (int64_t)c.capacity};
 }
 
+// Where a scheduler launch hands its summary to the host: BA_MAILBOX_BYTES of pinned, GPU-writable memory per
+// calling thread (allocated at the thread's first schedule, kept for the life of the process) and a ticket that
+// changes with every use.  The host then spins on the ticket instead of copying and synchronising the stream.
+struct Mailbox {
+    void *mem = nullptr;
+    uint32_t ticket = 0;
+    Mailbox() {
+        if (hipHostMalloc(&mem, BA_MAILBOX_BYTES, hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) mem = nullptr;
+        else memset(mem, 0, BA_MAILBOX_BYTES);
+    }
+};
+Mailbox &mailbox() {
+    static thread_local Mailbox m;
+    return m;
+}
+
 // The three metadata cases of the reference (cpp:17-44), resolved on the device.
 Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor &a2, const OptTensor &aO,
                        const OptTensor &M, const OptTensor &N, const OptTensor &K, bool use_cache = true) {
@@ -214,11 +230,23 @@ Schedule schedule_gemm(const Tensor &like, const OptTensor &a1, const OptTensor 
     const size_t bytes = ba_plan_bytes(nseg);
     s.plan = at::empty({(int64_t)bytes}, at::TensorOptions().dtype(at::kByte).device(like.device()));
     void *stream = current_stream(like);
-    check_status(ba_plan_gemm(s.plan.data_ptr(), bytes, nseg, mode, s.M.data_ptr<int64_t>(),
-                              s.N.data_ptr<int64_t>(), s.K.data_ptr<int64_t>(), s.accum1.data_ptr<int64_t>(),
-                              s.accum2.data_ptr<int64_t>(), s.accumOut.data_ptr<int64_t>(), stream),
-                 "ba_plan_gemm");
-    const int st = ba_plan_read(s.plan.data_ptr(), &s.info, stream);
+    Mailbox &mb = mailbox();
+    int st;
+    if (mb.mem) {
+        const uint32_t ticket = ++mb.ticket ? mb.ticket : ++mb.ticket;       // never 0, the mailbox's first content
+        check_status(ba_plan_gemm_notify(s.plan.data_ptr(), bytes, nseg, mode, s.M.data_ptr<int64_t>(),
+                                         s.N.data_ptr<int64_t>(), s.K.data_ptr<int64_t>(), s.accum1.data_ptr<int64_t>(),
+                                         s.accum2.data_ptr<int64_t>(), s.accumOut.data_ptr<int64_t>(), mb.mem, ticket,
+                                         stream),
+                     "ba_plan_gemm_notify");
+        st = ba_plan_wait(mb.mem, ticket, &s.info, 60 * 1000 * 1000);
+    } else {
+        check_status(ba_plan_gemm(s.plan.data_ptr(), bytes, nseg, mode, s.M.data_ptr<int64_t>(),
+                                  s.N.data_ptr<int64_t>(), s.K.data_ptr<int64_t>(), s.accum1.data_ptr<int64_t>(),
+                                  s.accum2.data_ptr<int64_t>(), s.accumOut.data_ptr<int64_t>(), stream),
+                     "ba_plan_gemm");
+        st = ba_plan_read(s.plan.data_ptr(), &s.info, stream);
+    }
     TORCH_CHECK(st != BA_ERR_BAD_METADATA, "segment metadata rejected: ", s.info.bad_segments,
                 " segment(s) have negative, oversized or inconsistent shapes / prefix sums");
     check_status(st, "ba_plan_read");
@@ -243,10 +271,20 @@ Schedule schedule_softmax(const Tensor &like, const Tensor &rows, const Tensor &
     const size_t bytes = ba_plan_bytes(nseg);
     s.plan = at::empty({(int64_t)bytes}, at::TensorOptions().dtype(at::kByte).device(like.device()));
     void *stream = current_stream(like);
-    check_status(ba_plan_softmax(s.plan.data_ptr(), bytes, nseg, rows.data_ptr<int64_t>(), cols.data_ptr<int64_t>(),
-                                 s.accumOut.data_ptr<int64_t>(), accum.has_value() ? 1 : 0, stream),
-                 "ba_plan_softmax");
-    const int st = ba_plan_read(s.plan.data_ptr(), &s.info, stream);
+    Mailbox &mb = mailbox();
+    int st;
+    if (mb.mem) {
+        const uint32_t ticket = ++mb.ticket ? mb.ticket : ++mb.ticket;
+        check_status(ba_plan_softmax_notify(s.plan.data_ptr(), bytes, nseg, rows.data_ptr<int64_t>(), cols.data_ptr<int64_t>(),
+                                            s.accumOut.data_ptr<int64_t>(), accum.has_value() ? 1 : 0, mb.mem, ticket, stream),
+                     "ba_plan_softmax_notify");
+        st = ba_plan_wait(mb.mem, ticket, &s.info, 60 * 1000 * 1000);
+    } else {
+        check_status(ba_plan_softmax(s.plan.data_ptr(), bytes, nseg, rows.data_ptr<int64_t>(), cols.data_ptr<int64_t>(),
+                                     s.accumOut.data_ptr<int64_t>(), accum.has_value() ? 1 : 0, stream),
+                     "ba_plan_softmax");
+        st = ba_plan_read(s.plan.data_ptr(), &s.info, stream);
+    }
     TORCH_CHECK(st != BA_ERR_BAD_METADATA, "segment metadata rejected: ", s.info.bad_segments,
                 " segment(s) have negative or oversized shapes or a prefix sum too small for them");
     check_status(st, "ba_plan_read");

@@ -134,6 +134,29 @@ int ba_plan_softmax(void *plan, size_t plan_bytes, int64_t nseg,
  * The results are identical either way. */
 int ba_plan_read(const void *plan, ba_plan_info *host_info, ba_stream_t stream);
 
+/* ba_plan_read without the library's own pinned buffer: the summary travels through `staging`, at least 256 bytes
+ * of host memory of the caller (pinned: no staging copy by the runtime), 16-byte aligned.  No counterpart in the
+ * reference (which reads its totals with .item(), csrc/cuda/spBlkGEMM.cu:996-998); for callers that want no
+ * allocation of any kind inside the library. */
+int ba_plan_read_into(const void *plan, ba_plan_info *host_info, void *staging, ba_stream_t stream);
+
+/* The schedulers once more, for calls whose metadata is new every time: in addition to the plan they write the
+ * summary into `mailbox` -- BA_MAILBOX_BYTES of host memory that the GPU can write and the CPU reads coherently
+ * (hipHostMalloc with hipHostMallocCoherent | hipHostMallocMapped), 16-byte aligned, caller-owned -- and behind it
+ * the 32-bit `ticket`.  ba_plan_wait spins on the host until the mailbox shows that ticket (timeout_us < 0: without
+ * limit; on a timeout BA_ERR_LAUNCH) and then returns what ba_plan_read would: no copy, no stream synchronisation.
+ * Use a ticket that differs from the one the mailbox showed last.  They replace the same reference code as
+ * ba_plan_gemm / ba_plan_softmax; the hand-over itself has no counterpart there. */
+#define BA_MAILBOX_BYTES 320
+int ba_plan_gemm_notify(void *plan, size_t plan_bytes, int64_t nseg, int mode,
+                        int64_t *MList, int64_t *NList, int64_t *KList,
+                        int64_t *accum1, int64_t *accum2, int64_t *accumOut,
+                        void *mailbox, uint32_t ticket, ba_stream_t stream);
+int ba_plan_softmax_notify(void *plan, size_t plan_bytes, int64_t nseg,
+                           const int64_t *rowList, const int64_t *colList,
+                           int64_t *accum, int accum_given, void *mailbox, uint32_t ticket, ba_stream_t stream);
+int ba_plan_wait(const void *mailbox, uint32_t ticket, ba_plan_info *host_info, int64_t timeout_us);
+
 /*
  * out[h, accumOut[g] + r*N_g + c] = sum_t A(h,g,r,t) * B(h,g,c,t), one rounding
  * to the operand dtype at the store.  Stands in for sparseBlockedGEMMLaunch

@@ -187,3 +187,23 @@ def test_main_strip_list_is_a_permutation_in_work_buckets(dev):
         else:
             want = np.arange(nseg)
         assert np.array_equal(lst["index"], want), nseg
+
+
+def test_summary_through_a_mailbox_and_through_caller_memory(dev):
+    # the scheduler hands the summary to the host in pinned memory (ticket behind it); the host spins, no copy and
+    # no stream synchronisation.  And ba_plan_read through a pinned buffer of the caller.  Both equal ba_plan_read.
+    rng = np.random.default_rng(12)
+    mailbox = torch.zeros(capi.MAILBOX_BYTES, dtype=torch.uint8).pin_memory()
+    staging = torch.zeros(256, dtype=torch.uint8).pin_memory()
+    for ticket, nseg in enumerate((5, 300, 2000), start=1):
+        M = rng.integers(0, 300, nseg); N = rng.integers(0, 300, nseg); K = 8 * rng.integers(0, 17, nseg)
+        Md, Nd, Kd = dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev)
+        acc = [torch.empty(nseg + 1, dtype=torch.int64, device=dev) for _ in range(3)]
+        plan = capi.plan_gemm(nseg, dev, Md, Nd, Kd, *acc, mode=capi.META_FROM_LISTS, mailbox=mailbox, ticket=ticket)
+        got = plan.wait(mailbox, ticket).as_dict()
+        want = plan.read().as_dict()
+        assert got == want and got["nseg"] == nseg
+        assert plan.read_into(staging).as_dict() == want
+    # a ticket nobody writes: the wait gives up
+    with pytest.raises(capi.BlockedAttentionError, match="launch"):
+        plan.wait(mailbox, 999, timeout_us=20_000)
