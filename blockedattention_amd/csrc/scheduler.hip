@@ -88,6 +88,11 @@ __device__ __forceinline__ int64_t isqrt64(int64_t v) {
 __device__ __forceinline__ bool derive_lists(int64_t mk, int64_t nk, int64_t mn, int64_t &m, int64_t &n,
                                              int64_t &k) {
     if (mk == 0 && nk == 0 && mn == 0) { m = n = k = 0; return true; }
+    // one empty dimension leaves one area: the product of the other two dimensions, whose split changes no
+    // result; it goes to the first of them whole
+    if (mk == 0 && mn == 0 && nk > 0) { m = 0; n = nk; k = 1; return true; }
+    if (nk == 0 && mn == 0 && mk > 0) { m = mk; n = 0; k = 1; return true; }
+    if (mk == 0 && nk == 0 && mn > 0) { m = mn; n = 1; k = 0; return true; }
     if (mk <= 0 || nk <= 0 || mn <= 0) return false;
     int64_t a = mk, b = nk;
     while (b) { const int64_t t = a % b; a = b; b = t; }
@@ -117,6 +122,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     __shared__ int64_t sScan64[16 * 3];
     __shared__ int32_t sScan32[16 * kNumScan];
     __shared__ int32_t sRed[kSchedWaves][6];
+    __shared__ int64_t sWeight[kSchedWaves];
 
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6), lane = lane_id();
@@ -127,6 +133,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     int32_t base32[kNumPrefix] = {};
     int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
     int32_t maxSmallN = 0, maxSmallM = 0;       // widest / tallest segment of the strip kernel's main launch
+    // Every scanned count of a segment is at most max(rows, strips x chunks): while the sum of these weights stays
+    // below 2^31, none of the int32 scans can overflow; a batch beyond that is rejected as a whole.
+    int64_t weight = 0;
     const bool offsets_given = a.mode != 0;   // prefix sums are inputs
 
     for (int64_t chunk = 0; chunk < nseg || chunk == 0; chunk += kSchedThreads) {
@@ -218,6 +227,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         for (int q = 0; q < kNumLists; ++q) v32[q] = cls == q ? 1 : 0;
         const bool wide_rows = mi >= 1 && ni > kRunCols;      // the softmax row kernel's, whatever the plan kind
         v32[kListRows] = wide_rows ? 1 : 0;
+        weight += max((int64_t)mi, (int64_t)strips * chunks) + 1;
         v32[kPfxGemm] = (mfma_ok && ni > kWaveCols) ? strips * chunks : 0;
         v32[kPfxStrip] = (mfma_ok && ni <= kWaveCols) ? strips : 0;
         v32[kPfxSplit] = (mfma_ok && ni > kWaveCols && ni <= kSplitCols) ? strips : 0;
@@ -298,6 +308,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     maxM = wave_max_nonneg(maxM); maxN = wave_max_nonneg(maxN); maxK = wave_max_nonneg(maxK);
     maxSmallN = wave_max_nonneg(maxSmallN); maxSmallM = wave_max_nonneg(maxSmallM);
     nbad = __builtin_amdgcn_readlane(wave_inclusive_scan(nbad), 63);
+#pragma unroll
+    for (int msk = 32; msk >= 1; msk >>= 1) weight += __shfl_xor(weight, msk);
+    if (lane == 0) sWeight[wave] = weight;
     if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; sRed[wave][4] = maxSmallN; sRed[wave][5] = maxSmallM; }
     __syncthreads();
 
@@ -314,8 +327,10 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             if (a.aO) a.aO[nseg] = DO;
         }
         int32_t rM = 0, rN = 0, rK = 0, rBad = 0, rSN = 0, rSM = 0;
+        int64_t total_weight = 0;
         for (int w = 0; w < kSchedWaves; ++w) {
             rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3];
+            total_weight += sWeight[w];
             rSN = max(rSN, sRed[w][4]); rSM = max(rSM, sRed[w][5]);
         }
         PlanHeader *h = pv.hdr;
@@ -328,7 +343,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         for (int q = 0; q < 12; ++q) h->totals[q] = q < kNumPrefix ? base32[q] : 0;
         h->max_M = rM; h->max_N = rN; h->max_K = rK;
         h->small_max_N = rSN; h->small_max_M = rSM;
-        h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0);
+        h->bad_segments = rBad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0) + (total_weight >= (int64_t(1) << 31) ? 1 : 0);
         h->run_errors = 0;
         h->att_blocks64 = base32[kPfxAtt64];
         h->att_blocks128 = base32[kPfxAtt128];

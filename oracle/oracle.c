@@ -67,7 +67,8 @@ static int64_t isqrt_i64(int64_t v) {
  * float32 and truncates; here it is exact integer arithmetic (the float route
  * can be off by one for large sizes, and the result must equal the lists that
  * generated the sums).  A segment whose three areas are all zero yields
- * (0,0,0).  Returns the number of segments whose areas are not consistent with
+ * (0,0,0); one with a single non-zero area has one empty dimension (the
+ * reference divides 0 by 0 there).  Returns the number of segments whose areas are not consistent with
  * any integer (M,N,K) (their lists are set to -1).
  */
 ORACLE_API int64_t oracle_accum_to_lists(const int64_t *accum1, const int64_t *accum2, const int64_t *accumOut,
@@ -78,6 +79,12 @@ ORACLE_API int64_t oracle_accum_to_lists(const int64_t *accum1, const int64_t *a
         int64_t nk = accum2[g + 1] - accum2[g];
         int64_t mn = accumOut[g + 1] - accumOut[g];
         if (mk == 0 && nk == 0 && mn == 0) { M[g] = N[g] = K[g] = 0; continue; }
+        /* One empty dimension leaves exactly one area: the sums fix only the product of the other two
+         * dimensions, and no result depends on how it splits (nothing is computed, or zeros fill M*N
+         * elements).  Convention: the whole product goes to the first of the two, the other is 1. */
+        if (mk == 0 && mn == 0 && nk > 0) { M[g] = 0; N[g] = nk; K[g] = 1; continue; }
+        if (nk == 0 && mn == 0 && mk > 0) { M[g] = mk; N[g] = 0; K[g] = 1; continue; }
+        if (mk == 0 && nk == 0 && mn > 0) { M[g] = mn; N[g] = 1; K[g] = 0; continue; }
         int ok = mk > 0 && nk > 0 && mn > 0;
         int64_t m = 0, n = 0, k = 0;
         if (ok) {

@@ -207,3 +207,29 @@ def test_summary_through_a_mailbox_and_through_caller_memory(dev):
     # a ticket nobody writes: the wait gives up
     with pytest.raises(capi.BlockedAttentionError, match="launch"):
         plan.wait(mailbox, 999, timeout_us=20_000)
+
+
+def test_prefix_sums_with_one_empty_dimension(dev):
+    # M = 0 (or N = 0, or K = 0) leaves a single non-zero area: the product of the other two dimensions, whose
+    # split changes no result.  The scheduler and the oracle take the same convention and accept the batch.
+    M = np.array([0, 5, 7, 0, 3]); N = np.array([4, 0, 6, 0, 2]); K = np.array([8, 8, 0, 0, 16])
+    a1, a2, ao = oracle.lists_to_accum(M, N, K)
+    Mo, No, Ko, bad = oracle.accum_to_lists(a1, a2, ao)
+    assert bad == 0
+    assert np.array_equal(Mo * Ko, M * K) and np.array_equal(No * Ko, N * K) and np.array_equal(Mo * No, M * N)
+    lists = [torch.empty(5, dtype=torch.int64, device=dev) for _ in range(3)]
+    plan = capi.plan_gemm(5, dev, *lists, dev_i64(a1, dev), dev_i64(a2, dev), dev_i64(ao, dev), mode=capi.META_FROM_ACCUM)
+    info = plan.read()
+    assert info.bad_segments == 0
+    got = [t.cpu().numpy() for t in lists]
+    assert np.array_equal(got[0], Mo) and np.array_equal(got[1], No) and np.array_equal(got[2], Ko)
+
+
+def test_batches_beyond_the_32_bit_work_counts_are_rejected(dev):
+    # three segments of 2^30 - 1 rows each: every one is admissible, their row count together is not
+    big = (1 << 30) - 1
+    M = np.array([big, big, big]); N = np.array([1, 1, 1]); K = np.array([0, 0, 0])
+    plan = make_plan(dev, M, N, K, read=False)
+    assert plan.read(raise_on_bad=False).bad_segments >= 1
+    plan = make_plan(dev, M[:1], N[:1], K[:1], read=False)
+    assert plan.read(raise_on_bad=False).bad_segments == 0

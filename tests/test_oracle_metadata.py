@@ -62,10 +62,14 @@ def test_accum_to_lists_large_sizes_exact():
 
 def test_accum_to_lists_zero_and_inconsistent_segments():
     a1 = np.array([0, 0, 6, 6]); a2 = np.array([0, 0, 10, 13]); ao = np.array([0, 0, 15, 15])
-    # segment 0: all areas zero -> (0,0,0); segment 1: (3,5,2); segment 2: mk=0, nk=3, mn=0 -> inconsistent
+    # segment 0: all areas zero -> (0,0,0); segment 1: (3,5,2); segment 2: mk=0, nk=3, mn=0 -> no rows, and the
+    # three elements of B go to N whole (their split into N x K changes nothing)
     m, n, k, bad = oracle.accum_to_lists(a1, a2, ao)
+    assert bad == 0
+    assert (m[0], n[0], k[0]) == (0, 0, 0) and (m[1], n[1], k[1]) == (3, 5, 2) and (m[2], n[2], k[2]) == (0, 3, 1)
+    # two non-zero areas and one zero: no triple at all
+    _, _, _, bad = oracle.accum_to_lists([0, 6], [0, 10], [0, 0])
     assert bad == 1
-    assert (m[0], n[0], k[0]) == (0, 0, 0) and (m[1], n[1], k[1]) == (3, 5, 2) and m[2] == -1
     # areas that match no integer triple
     _, _, _, bad = oracle.accum_to_lists([0, 6], [0, 10], [0, 14])
     assert bad == 1
