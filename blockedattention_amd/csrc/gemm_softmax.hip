@@ -768,7 +768,9 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     // workgroups per compute unit; the wide build holds two (64 KiB window) or three (registers), and one round of
     // resident workgroups that loop over their strips beats several rounds of short ones (non-square 512-segment
     // batch: 17.9 us with one workgroup per segment, 19.7 us with four).
+    static const int z_env = [] { const char *e = getenv("BLOCKEDATTN_STRIP_Z"); return e ? atoi(e) : 0; }();
     auto strip_z = [&](int64_t slots, int64_t tallest, int per_cu) {
+        if (z_env > 0) return (int64_t)z_env;
         if (!info) return (int64_t)2;
         const int64_t groups = ceil_div(ceil_div(std::max<int64_t>(tallest, 1), kStripRows), kSegWaves);
         const int64_t want = ceil_div((int64_t)cus * per_cu, std::max<int64_t>(1, slots * (int64_t)H));
