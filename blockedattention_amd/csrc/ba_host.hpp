@@ -37,6 +37,8 @@ struct RunArgs {
     int ride_slots;   // ride_slots x H x ride_z workgroups, slot fastest
     int ride_z;
     int both_split;   // with kFlagSmallToo: length of the launch's own list; slot s >= both_split is entry s - both_split of the small list
+    int mini_first;   // strip kernel: first slot of the mini entries of the main list (0: the launch carries none) ...
+    int mini_solo;    // ... 1: four to a workgroup, one wavefront each (64 KiB window); 0: one workgroup each
 };
 
 int launch_schedule(void *plan, size_t plan_bytes, int64_t nseg, int mode, int kind, int64_t *M, int64_t *N,

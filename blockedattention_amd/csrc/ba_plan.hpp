@@ -65,8 +65,21 @@ enum PrefixKind {
     kPfxSlow = 11,  // ceil(M/16) for segments the 16-byte operand loads cannot serve
     kPfxAtt64 = 12,   // GEMM plans: ceil(M/64) for every segment with rows (one-pass attention, any-layout GEMM)
     kPfxAtt128 = 13,  // the same in row blocks of 128
-    kNumPrefix = 14
+    kPfxMini = 14,    // 1 for a segment of the strip kernel's main list that is small enough for one wavefront
+    kNumPrefix = 15
 };
+
+// "Mini" segments: strip-class segments of at most 64 rows whose B_g needs at most kMiniBlocks LDS blocks and at most
+// eight column tiles.  One wavefront can take such a segment on its own (a quarter of a 64 KiB window), so four of
+// them share a workgroup where the launch has that window.  They belong to the main strip list, but are kept
+// apart from its other entries: entry k of them sits at position cap - 1 - k of that list's array (from the end
+// backwards), totals[kListSmall] counts the others, PlanHeader::mini_count these.
+constexpr int kMiniBlocks = 16;
+constexpr int kMiniRows = 64;
+__host__ __device__ inline bool mini_shape(int M, int N, int K) {
+    const int b = strip_blocks(N, K);
+    return M >= 1 && M <= kMiniRows && b >= 1 && b <= kMiniBlocks && fast_strip_tiles(N) <= 8;
+}
 constexpr int kMailboxTicket = 256;   // byte offset of the ticket word in a scheduler mailbox (behind the header copy)
 constexpr int kAttBlockRows = 64;   // kPfxAtt64 counts blocks of this many rows, kPfxAtt128 of twice as many
 
@@ -89,7 +102,8 @@ struct PlanHeader {
     int32_t run_errors;      // bumped by kernels that refuse to run
     int32_t small_max_N, small_max_M;   // maxima over the segments of the strip kernel's main launch
     int32_t att_blocks64, att_blocks128;   // totals of kPfxAtt64 / kPfxAtt128: the one-pass attention's row blocks per head
-    int32_t pad_[19];
+    int32_t mini_count;      // total of kPfxMini
+    int32_t pad_[18];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 

@@ -122,6 +122,7 @@ static int info_from_header(const PlanHeader &h, ba_plan_info *info) {
     info->small_max_M = h.small_max_M;
     info->att_blocks64 = h.att_blocks64;
     info->att_blocks128 = h.att_blocks128;
+    info->list_mini = h.mini_count;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 

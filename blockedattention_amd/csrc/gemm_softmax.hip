@@ -426,9 +426,14 @@ __device__ __forceinline__ void strips_from_lds_dispatch(int nt, const Seg &s, c
 // that read one operand together hold the same piece of rows G apart, i.e. of sixteen different slots
 // j, they fall into sixteen different bank groups.  The run [N-G, N) of the lane at the ragged end
 // (and of the lanes after it) is copied once more, unpermuted, behind the image and read from there.
-template <int DT, int G, bool FUSED, bool F32OUT, int NAT>
-__device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, unsigned char *lds, int wave,
+// SOLO: the calling wavefront has the segment and the LDS it is given to itself (a mini segment, see mini_shape):
+// it fills alone, waits for its own loads and passes no barrier, so the wavefronts of a workgroup can work on
+// different segments, each in its own code.
+template <int DT, int G, bool FUSED, bool F32OUT, int NAT, bool SOLO = false>
+__device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, unsigned char *lds, int wave_in,
                                              int first_strip, int strip_step) {
+    constexpr int kFillWaves = SOLO ? 1 : kSegWaves;
+    const int wave = SOLO ? 0 : wave_in;
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
     const int K = s.K, N = s.N, M = s.M;
     const int nks = (K + 31) >> 5;
@@ -462,7 +467,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         const int brow0 = owner ? col0 : N - 1;
         const int bstep = owner ? 1 : 0;
         const int nblocks = nks * G;
-        for (int b = wave; b < nblocks; b += kSegWaves) {
+        for (int b = wave; b < nblocks; b += kFillWaves) {
             const int ks = b / G, g = b - ks * G;
             const int row = brow0 + bstep * g;
             int kk = ks * 32 + rg * 8;
@@ -481,7 +486,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         // last piece into positions nobody reads, so the image takes whole KiB and the copy of the ragged
         // run starts on the next KiB.
         const int total = N * kPieces, padded = (total + 63) & ~63;
-        for (int p0 = wave * 64; p0 < padded; p0 += kSegWaves * 64) {
+        for (int p0 = wave * 64; p0 < padded; p0 += kFillWaves * 64) {
             const int p = p0 + lane, w = p >> 4;
             const int key = ((NAT == 1 ? 2 * w : w) / G) & 15;
             const int piece = min((p & ~15) | ((p & 15) ^ key), total - 1);
@@ -491,7 +496,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         unsigned char *tail = lds + padded * 16;
         const int tail_pieces = G * kPieces;
         const int tail_key = J & 15;         // no lane with a full run uses this key: the copy's readers collide with none
-        for (int p0 = wave * 64; p0 < tail_pieces; p0 += kSegWaves * 64) {
+        for (int p0 = wave * 64; p0 < tail_pieces; p0 += kFillWaves * 64) {
             const int q = p0 + lane;
             const int p = min((q & ~15) | ((q & 15) ^ tail_key), tail_pieces - 1);
             __builtin_amdgcn_global_load_lds(
@@ -512,7 +517,7 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
         for (int g = 0; g < G; ++g) w[g] = (j < J || (j == J && g >= G - v)) ? 1.f : 0.f;
     }
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+    if constexpr (!SOLO) __syncthreads();
 
     // address of the operand of column tile g, k-step ks (g, ks: unrolled constants)
     auto operand = [&](int g, int ks) -> const unsigned char * {
@@ -610,6 +615,24 @@ __device__ __forceinline__ void strips_exact_dispatch(int tiles, const Seg &s, c
 #undef BA_EXACT
 }
 
+// One wavefront, one mini segment, `lds` = the wavefront's own kMiniBlocks KiB.
+template <int DT, bool FUSED, bool F32OUT>
+__device__ __forceinline__ void strips_solo_dispatch(int tiles, const Seg &s, const RunArgs &a, unsigned char *lds) {
+    const int pieces = s.N * (s.K >> 3);
+    const bool image_fits = (((pieces + 63) & ~63) + ((tiles * (s.K >> 3) + 63) & ~63)) * 16 <= kMiniBlocks * kLdsBlockBytes;
+#define BA_SOLO(G_)                                                                                        \
+    case G_:                                                                                               \
+        if (s.K == 64 && image_fits) strips_exact<DT, G_, FUSED, F32OUT, 1, true>(s, a, lds, 0, 0, 1);     \
+        else if (s.K == 128 && image_fits) strips_exact<DT, G_, FUSED, F32OUT, 2, true>(s, a, lds, 0, 0, 1); \
+        else strips_exact<DT, G_, FUSED, F32OUT, 0, true>(s, a, lds, 0, 0, 1);                             \
+        break;
+    switch (tiles) {
+        BA_SOLO(2) BA_SOLO(4) BA_SOLO(6) BA_SOLO(8)
+        default: break;
+    }
+#undef BA_SOLO
+}
+
 // ------------------------------------------------------------------ kernels
 // segment_kernel   grid (segment, head, z): one workgroup per segment and head;
 //                  its wavefronts take the segment's 16-row strips (N <= 256),
@@ -695,12 +718,35 @@ __global__ __launch_bounds__(kSegThreads, MAXNT <= 8 ? 4 : 2) void strip_kernel(
         bz = lin / ((unsigned)a.ride_slots * (unsigned)a.H);
         gz = (unsigned)a.ride_z;
     }
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
+    const int64_t h = by;
+    if (a.mini_first > 0 && bx >= (unsigned)a.mini_first) {
+        // The mini entries of the main list (kept at the end of its array, backwards): four to a workgroup, one
+        // wavefront and a quarter of the 64 KiB window each, or one workgroup each where the window is smaller.
+        const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
+        const int count = hdr->mini_count;
+        const bool ok = header_ok(a);
+        const int wave = uniform((int)(threadIdx.x >> 6));
+        const int k = a.mini_solo ? 4 * (int)(bx - (unsigned)a.mini_first) + wave : (int)(bx - (unsigned)a.mini_first);
+        // header, count and record are fetched together (the record from a position that exists whatever k is)
+        const int64_t cap = plan_cap(a.nseg);
+        const SegRec r = load_rec(pv.recs + (int64_t)(kListSmall + 1) * cap, (int)(cap - 1 - min((int64_t)k, cap - 1)));
+        if (!ok || k >= count || bz != 0) return;       // (a plan that does not match is reported by the launch's other blocks)
+        Seg s;
+        s.M = r.M; s.N = r.N; s.K = r.K;
+        s.kind = r.kind; s.index = r.index; s.packLen = r.packLen;
+        s.a = h * a.Dm1 + r.off1; s.b = h * a.Dm2 + r.off2; s.o = h * a.Dout + r.offO;
+        const int tiles = fast_strip_tiles(s.N);
+        if (s.kind != kSegStrip || !mini_shape(s.M, s.N, s.K) || tiles > MAXNT) return;
+        if (a.mini_solo) strips_solo_dispatch<DT, FUSED, F32OUT>(tiles, s, a, lds + wave * (kMiniBlocks * kLdsBlockBytes));
+        else if (strip_blocks(s.N, s.K) <= a.lds_blocks)
+            strips_exact_dispatch<DT, FUSED, F32OUT, MAXNT>(tiles, s, a, lds, wave, wave, kSegWaves);
+        return;
+    }
     if ((a.flags & kFlagSmallToo) && bx >= (unsigned)a.both_split) {
         bx -= (unsigned)a.both_split;
         a.list = kListSmall;
     }
-    const PlanRO pv = plan_ro(a.plan, a.nseg);
-    const int64_t h = by;
     // header and record are fetched together; nothing waits on the header alone
     const bool ok = header_ok(a);
     bool valid;
@@ -762,6 +808,7 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     const int64_t n_big = !mfma_ok ? 0 : info ? info->list_big : nseg;
     const int64_t n_tile = !mfma_ok ? 0 : info ? info->list_tile : nseg;
     const int64_t n_rest = !mfma_ok ? nseg : info ? info->list_rest : nseg;
+    const int64_t n_mini = !mfma_ok ? 0 : info ? info->list_mini : nseg;    // part of the main strip list, kept apart
     const bool lean = info && info->max_N <= 128;
     // z: enough workgroups to fill the machine, at most one per kSegWaves strips of the tallest segment.  The
     // narrow build (up to eight column tiles, four to five workgroups resident per compute unit) aims at eight
@@ -778,7 +825,7 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     };
     // the rest list is nothing but pack leaders: the first strip launch takes them along
     const bool packs_ride = info && mfma_ok && n_rest > 0 && n_rest == info->pack_items && info->slow_items == 0 &&
-                            (n_small > 0 || n_big > 0);
+                            (n_small > 0 || n_big > 0 || n_mini > 0);
     bool packs_taken = false;
     // a modest amount of tile-kernel work rides in the strip kernel's 64 KiB launch (same LDS, same
     // residency) instead of following it; large tile work keeps its own die-aware launch
@@ -794,9 +841,13 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
     static const int merge_env = [] { const char *e = getenv("BLOCKEDATTN_MERGE_STRIPS"); return e ? atoi(e) : -1; }();
     const bool merge = info && n_small > 0 && n_big > 0 &&
                        (merge_env >= 0 ? merge_env != 0 : info->small_max_N > 128 || (n_small + n_big) * (int64_t)H <= 4096);
+    // The mini entries ride in ONE of the strip launches: the merged one, else the main launch if it has entries
+    // of its own, else the 64 KiB launch, else a main launch for them alone.
+    const int mini_pass = n_mini <= 0 ? -1 : merge ? 1 : n_small > 0 ? 0 : n_big > 0 ? 1 : 0;
+    static const int solo_env = [] { const char *e = getenv("BLOCKEDATTN_MINI_SOLO"); return e ? atoi(e) : 1; }();
     for (int pass = 0; pass < 2; ++pass) {
         int64_t slots = pass == 0 ? n_small : n_big;
-        if (slots <= 0 || (merge && pass == 0)) continue;
+        if ((slots <= 0 && pass != mini_pass) || (merge && pass == 0)) continue;
         RunArgs fa = args;
         if (merge) {
             fa.flags |= kFlagSmallToo;
@@ -826,6 +877,13 @@ static int launch_set(int dtype, const RunArgs &args_in, int64_t nseg, const ba_
             const int64_t nks = ceil_div(std::max<int64_t>(info->max_K, 1), 32);
             fa.lds_blocks = (int)std::min<int64_t>(kFastBlocks, nt * nks);
             lean_pass = info->small_max_N <= 128;
+        }
+        if (pass == mini_pass) {
+            // four mini segments to a workgroup where the window has a quarter for each of them
+            fa.mini_first = (int)std::max<int64_t>(slots, 1);
+            fa.mini_solo = solo_env && info && fa.lds_blocks >= 4 * kMiniBlocks ? 1 : 0;
+            slots = fa.mini_first + (fa.mini_solo ? ceil_div(n_mini, kSegWaves) : n_mini);
+            if (ride) fa.ride_slots = (int)slots;
         }
         const int64_t tallest = !info ? 0 : pass == 0 ? info->small_max_M : info->max_M;
         const dim3 grid((unsigned)slots, H, (unsigned)strip_z(slots, tallest, lean_pass ? 8 : pass == 0 ? 3 : 2));

@@ -222,9 +222,11 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
                                  : ni <= kWaveCols ? kSegStrip
                                  : ni <= kSplitCols ? kSegSplit : kSegWide;
         const int cls = a.kind == 0 ? launch_class(seg_kind, mi, ni, ki) : -1;
+        const bool mini = cls == kListSmall && mini_shape(mi, ni, ki);     // kept apart from the list's other entries
         int32_t v32[kNumScan], t32[kNumScan];
 #pragma unroll
-        for (int q = 0; q < kNumLists; ++q) v32[q] = cls == q ? 1 : 0;
+        for (int q = 0; q < kNumLists; ++q) v32[q] = (cls == q && !mini) ? 1 : 0;
+        v32[kPfxMini] = mini ? 1 : 0;
         const bool wide_rows = mi >= 1 && ni > kRunCols;      // the softmax row kernel's, whatever the plan kind
         v32[kListRows] = wide_rows ? 1 : 0;
         weight += max((int64_t)mi, (int64_t)strips * chunks) + 1;
@@ -247,7 +249,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         // tiles / 8, clipped): workgroups that start together then take about equally long and the longest
         // start first (256 segments x 8 heads of 32..128 rows: fused kernel 16.1 -> 15.4 us).  One counter of
         // 16 bits per bucket (a pass holds at most 1024 segments), two to a scanned word.
-        const int bucket = cls == kListSmall ? min(kSmallBuckets - 1, min(strips, 64) * fast_strip_tiles(min(ni, 256)) / 8) : -1;
+        const int bucket = (cls == kListSmall && !mini) ? min(kSmallBuckets - 1, min(strips, 64) * fast_strip_tiles(min(ni, 256)) / 8) : -1;
         if constexpr (kBucketed) {
 #pragma unroll
             for (int wd = 0; wd < kSmallBuckets / 2; ++wd)
@@ -274,7 +276,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             pv.recs[g] = rec;
 #pragma unroll
             for (int q = 0; q < kNumLists; ++q)          // v32 now holds the exclusive scans
-                if (cls == q) pv.list[q][base32[q] + (q == kListSmall ? small_pos : v32[q])] = rec;
+                if (cls == q && !mini) pv.list[q][base32[q] + (q == kListSmall ? small_pos : v32[q])] = rec;
+            if (mini) pv.list[kListSmall][plan_cap(nseg) - 1 - (base32[kPfxMini] + v32[kPfxMini])] = rec;
             if (wide_rows) pv.list[kListRows][base32[kListRows] + v32[kListRows]] = rec;
             if (a.kind == 0) {
                 plan_rowblocks(a.plan, nseg, 0)[g] = base32[kPfxAtt64] + v32[kPfxAtt64];
@@ -347,6 +350,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->run_errors = 0;
         h->att_blocks64 = base32[kPfxAtt64];
         h->att_blocks128 = base32[kPfxAtt128];
+        h->mini_count = base32[kPfxMini];
         plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
         plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
         if (a.mailbox) {

@@ -80,9 +80,12 @@ typedef struct ba_plan_info {
     int32_t small_max_N;    /* widest segment of the strip kernel's main launch */
     int32_t small_max_M;    /* tallest segment of the strip kernel's main launch */
     int32_t list_rows;      /* softmax row kernel: segments with N > 256 (GEMM and softmax plans) */
-    /* one-pass attention, GEMM plans: row blocks of 64 and of 128 rows per head, summed over the segments
-     * with M >= 1 and K >= 1 whatever their N (a segment without keys still has its output rows zeroed) */
+    /* GEMM plans: row blocks of 64 and of 128 rows per head, summed over the segments with M >= 1 whatever
+     * their N and K (one-pass attention: a segment without keys still has its output rows zeroed) */
     int32_t att_blocks64, att_blocks128;
+    /* segments of the strip kernel's main launch that one wavefront can take alone (at most 64 rows, B_g of
+     * at most 16 KiB); list_small counts the others */
+    int32_t list_mini;
 } ba_plan_info;
 
 const char *ba_status_string(int status);

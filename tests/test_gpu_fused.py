@@ -96,11 +96,13 @@ def test_work_lists_match_the_shape_rules(dev):
         tiles = 2 * ((w.N + 31) // 32); nks = (w.K + 31) // 32
         blocks = np.where((w.N >= 2) & (w.N <= 256) & (nks >= 1) & (nks <= 4), tiles * nks, 0)
         aligned = (w.K % 8 == 0)                       # offsets of these configurations are multiples of 8 with K
-        packed = i.list_small + i.list_big + i.list_tile + i.list_rest
+        packed = i.list_small + i.list_mini + i.list_big + i.list_tile + i.list_rest
         small = int(((blocks >= 1) & (blocks <= 32) & aligned).sum())
         big = int(((blocks > 32) & (blocks <= 64) & aligned).sum())
         assert i.list_big == big, cfg
-        assert i.list_small <= small and small - i.list_small <= 2 * i.pack_items * 8, cfg   # packs take tiny ones
+        main = i.list_small + i.list_mini                # the main strip list: its mini entries are counted apart
+        assert main <= small and small - main <= 2 * i.pack_items * 8, cfg   # packs take tiny ones
+        assert i.list_mini <= int(((w.M <= 64) & (blocks >= 1) & (blocks <= 16) & (tiles <= 8) & aligned).sum()), cfg
         assert i.list_tile == int(((w.N > 256) | ((w.N >= 128) & (blocks == 0))).sum()), cfg
         assert packed <= w.nseg
         assert i.list_rows == int(((w.N > 256) & (w.M >= 1)).sum()), cfg     # the softmax row kernel's list
@@ -129,13 +131,14 @@ def test_both_strip_lists_merged_and_separate(dev):
             K[:8] = 32; N[:8] = 250                      # 16 tiles x 1 k-step: the 32 KiB list, wider than 128
         N[-1] = 300; M[-1] = 130                         # one tile-kernel segment rides along
         return M, N, K
-    for nseg, heads, wide_small in ((40, 2, False), (40, 2, True), (600, 7, False), (600, 7, True)):
+    for nseg, heads, wide_small in ((40, 2, False), (40, 2, True), (1200, 7, False), (1200, 7, True)):
         M, N, K = batch(nseg, wide_small)
         plan = run_all(dev, M, N, K, heads, torch.bfloat16, 0.09, seed=nseg + heads, check_softmax=False)
         i = plan.info
         assert i.list_small > 0 and i.list_big > 0 and i.list_tile == 1
         assert (i.small_max_N > 128) == wide_small
-        assert ((i.list_small + i.list_big) * heads > 4096) == (nseg == 600)
+        assert i.list_mini > 0                           # narrow segments of few rows: one wavefront each
+        assert ((i.list_small + i.list_big) * heads > 4096) == (nseg == 1200)
 
 
 def test_more_list_entries_than_the_second_grid_dimension_holds(dev):
@@ -145,4 +148,4 @@ def test_more_list_entries_than_the_second_grid_dimension_holds(dev):
     nseg = 66000
     M = rng.integers(17, 25, nseg); N = rng.integers(17, 25, nseg); K = np.full(nseg, 8)
     plan = run_all(dev, M, N, K, 2, torch.float16, 0.3, seed=2)
-    assert plan.info.list_small == nseg
+    assert plan.info.list_small + plan.info.list_mini == nseg and plan.info.list_mini > 0

@@ -165,27 +165,41 @@ def test_row_block_prefixes_of_the_attention_work_list(dev):
             assert np.array_equal(got, want), (nseg, rows)
 
 
+def _mini(M, N, K):
+    tiles = 2 * ((N + 31) // 32); blocks = tiles * ((K + 31) // 32)
+    return (M >= 1) & (M <= 64) & (N >= 2) & (blocks >= 1) & (blocks <= 16) & (tiles <= 8)
+
+
 def test_main_strip_list_is_a_permutation_in_work_buckets(dev):
     # Batches of 65 to 256 segments keep the main strip launch's list in eight buckets of decreasing work
     # (16-row strips x column tiles / 8, clipped at 7), in segment order inside a bucket; every other batch
-    # keeps segment order.  Either way the list holds each of its segments exactly once.
+    # keeps segment order.  The mini segments of the list (at most 64 rows, B_g of at most 16 KiB, at most eight
+    # column tiles) are kept apart, from the end of the list's array backwards, in segment order.  Together the
+    # two parts hold each segment of the list exactly once.
     rec = np.dtype([("o1", "<i8"), ("o2", "<i8"), ("oo", "<i8"), ("M", "<i4"), ("N", "<i4"), ("K", "<i4"),
                     ("pack", "<i4"), ("kind", "<i4"), ("index", "<i4")])
     rng = np.random.default_rng(5)
     for nseg in (40, 200, 256, 300):
         M = rng.integers(17, 130, nseg); N = rng.integers(17, 130, nseg); K = np.full(nseg, 64)
         plan = make_plan(dev, M, N, K)
-        assert plan.info.list_small == nseg
+        mini = _mini(M, N, K)
+        assert 0 < mini.sum() < nseg
+        assert plan.info.list_small == nseg - mini.sum() and plan.info.list_mini == mini.sum()
         cap = (nseg + 4) & ~3
         raw = plan.buf.cpu().numpy()
-        lst = raw[256 + cap * 48: 256 + cap * 48 + nseg * 48].view(rec)
-        assert sorted(lst["index"].tolist()) == list(range(nseg))
-        assert np.array_equal(lst["M"], M[lst["index"]]) and np.array_equal(lst["N"], N[lst["index"]])
-        bucket = np.minimum(7, ((M + 15) // 16) * (2 * ((N + 31) // 32)) // 8)
+        arr = raw[256 + cap * 48: 256 + 2 * cap * 48].view(rec)
+        lst = arr[:plan.info.list_small]
+        tail = arr[::-1][:plan.info.list_mini]
+        assert sorted(lst["index"].tolist() + tail["index"].tolist()) == list(range(nseg))
+        assert np.array_equal(tail["index"], np.nonzero(mini)[0])
+        for part in (lst, tail):
+            assert np.array_equal(part["M"], M[part["index"]]) and np.array_equal(part["N"], N[part["index"]])
+        others = np.nonzero(~mini)[0]
+        bucket = np.minimum(7, ((M + 15) // 16) * (2 * ((N + 31) // 32)) // 8)[others]
         if 64 < nseg <= 256:
-            want = np.argsort(-bucket, kind="stable")
+            want = others[np.argsort(-bucket, kind="stable")]
         else:
-            want = np.arange(nseg)
+            want = others
         assert np.array_equal(lst["index"], want), nseg
 
 
