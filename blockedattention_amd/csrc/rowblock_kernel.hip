@@ -40,6 +40,7 @@ namespace ba {
 constexpr int kRbWaves = 8;
 constexpr int kRbThreads = 64 * kRbWaves;
 constexpr int kRbWaveRows = 32;
+constexpr int kRbRT = kRbWaveRows / 16;                 // MFMA row tiles per wavefront
 constexpr int kRbRows = kRbWaves * kRbWaveRows;          // 256 rows per workgroup
 constexpr int kRbCols = 64;                               // columns per chunk
 constexpr int kRbRowBytes = 256;                          // one row of B_g in LDS: 128 k
@@ -201,9 +202,9 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
         const int row0 = rb * kRbRows + wave * kRbWaveRows;     // first row of this wavefront
         const bool active = row0 < M;
         // ---- A fragments [rt][ks]: row 16 rt + j, k = 32 ks + 8 rg ..
-        u32x4 af[kRT][KS];
+        u32x4 af[kRbRT][KS];
 #pragma unroll
-        for (int rt = 0; rt < kRT; ++rt) {
+        for (int rt = 0; rt < kRbRT; ++rt) {
             const int voff = ((row0 + 16 * rt + j) * K + rg * 8) * 2;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -249,12 +250,12 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
             // every iteration, stores in flight included.
             wait_vm<0>();
             // per-row state: sweep 1: ref = -R c (bias of the exponent) and the running sum; sweep 2: ref = -R c - log2(sum)
-            float ref[kRT][4], sum[kRT][4], rmax[kRT][4];
+            float ref[kRbRT][4], sum[kRbRT][4], rmax[kRbRT][4];
 #pragma unroll
-            for (int rt = 0; rt < kRT; ++rt)
+            for (int rt = 0; rt < kRbRT; ++rt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) { ref[rt][i] = 0.f; sum[rt][i] = 0.f; rmax[rt][i] = -3.0e38f; }
-            f32x4 acc[2][kRT][4];
+            f32x4 acc[2][kRbRT][4];
             bool restart = false;
 
             // -------- out of the ring: one line-aligned 128-byte window per row and chunk.  Interior chunks: every
@@ -406,7 +407,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                 constexpr int b = decltype(buf_c)::value;
                 const int cb = cbi * kRbCols;
 #pragma unroll
-                for (int rt = 0; rt < kRT; ++rt) {
+                for (int rt = 0; rt < kRbRT; ++rt) {
                     float mx[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
@@ -431,7 +432,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
             auto finish_stats = [&]() __attribute__((always_inline)) {
                 bool bad = false;
 #pragma unroll
-                for (int rt = 0; rt < kRT; ++rt) {
+                for (int rt = 0; rt < kRbRT; ++rt) {
                     float sm[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) sm[i] = sum[rt][i];
