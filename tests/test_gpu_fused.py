@@ -149,3 +149,28 @@ def test_more_list_entries_than_the_second_grid_dimension_holds(dev):
     M = rng.integers(17, 25, nseg); N = rng.integers(17, 25, nseg); K = np.full(nseg, 8)
     plan = run_all(dev, M, N, K, 2, torch.float16, 0.3, seed=2)
     assert plan.info.list_small + plan.info.list_mini == nseg and plan.info.list_mini > 0
+
+
+def test_mini_segments_alone_and_among_others(dev):
+    # Segments of at most 64 rows whose B_g takes at most 16 KiB: one wavefront each, four to a workgroup where the
+    # launch has the 64 KiB window (a wide segment in the batch), one workgroup each otherwise.  Every boundary of the
+    # class: 64 / 65 rows, 16 / 17 operand blocks, every tile count up to eight, every B_g layout (K = 64, 128, other),
+    # ragged columns, one row, groups of four that are not full.
+    rng = np.random.default_rng(31)
+    M = np.array([64, 65, 1, 16, 17, 33, 48, 64, 5, 64, 20, 64, 31])
+    N = np.array([64, 64, 2, 33, 127, 128, 96, 129, 250, 17, 64, 61, 256])
+    K = np.array([128, 128, 128, 64, 64, 64, 72, 48, 32, 128, 104, 120, 32])
+    wide = (np.array([200]), np.array([256]), np.array([128]))        # B_g of 64 KiB: the launch gets the wide window
+    for extra, heads, dtype, scale in ((None, 3, torch.float16, 0.2), (wide, 2, torch.bfloat16, -0.1),
+                                       (wide, 5, torch.float16, 0.0)):
+        m, n, k = (M, N, K) if extra is None else tuple(np.concatenate([a, b]) for a, b in zip((M, N, K), extra))
+        plan = run_all(dev, m, n, k, heads, dtype, scale, seed=3)
+        i = plan.info
+        assert i.list_mini == 8 and i.list_big == (0 if extra is None else 1)
+        run_all(dev, m, n, k, heads, dtype, scale, seed=4, summary=False)
+    # many of them, a count that is not a multiple of four, among two wide segments
+    nseg = 203
+    m = rng.integers(1, 65, nseg); n = rng.integers(2, 65, nseg); k = np.full(nseg, 128)
+    m[[7, 150]] = 180; n[[7, 150]] = 250
+    plan = run_all(dev, m, n, k, 3, torch.bfloat16, 128 ** -0.5, seed=5)
+    assert plan.info.list_mini >= 150 and plan.info.list_big == 2
