@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 #include "ba_device.hpp"
 #include "ba_gemm_common.hpp"
@@ -37,9 +38,31 @@ constexpr int kAttWaves = kAttThreads / 64;
 constexpr int kAttKeys = 64;                          // keys per block
 constexpr int kAttRows = 16 * kAttWaves;              // queries per workgroup round
 static_assert(kAttRows == kAttBlockRows, "the plan's row-block prefixes count blocks of kAttRows and 2 kAttRows");
-constexpr int kAttPitchV = kAttKeys * 2 + 8;          // bytes per LDS row of transposed values.  An LDS access
-// serves 16 lanes x 8 bytes at a time; the 8-byte skew puts the sixteen rows 16 t + j that an operand read
-// touches in sixteen different 8-byte bank groups, and a staging write covers one row's 128 bytes.
+constexpr int kAttPitchV = kAttKeys * 2 + 16;         // bytes per LDS row of transposed values: the sixteen rows
+// 16 t + j that an operand read (16 bytes per lane) touches start in sixteen different groups of four banks, and
+// a staging write (8 bytes per lane, 32 lanes at a time) covers two rows that lie 32 banks apart.
+constexpr int kAttRing = 6;                           // LDS operand reads in flight per wavefront
+
+// LDS operand reads as inline assembly, so that kAttRing of them are in flight under the matrix instructions
+// (left to itself the compiler, short of registers, issues each read right before its use and every matrix
+// instruction waits a full LDS round trip).  The compiler does not count these reads: lds_wait<n> waits until at
+// most n of them are outstanding and hands the register on, so the use cannot move above the wait.  Counting is
+// conservative when other LDS or scalar loads are in flight: the counter is then higher, the wait longer.
+template <int OFF> __device__ __forceinline__ void lds_read128(u32x4 &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int N> __device__ __forceinline__ void lds_wait(u32x4 &x) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N) : "memory");
+}
+template <typename F, int... I> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+__device__ __forceinline__ uint32_t lds_offset(const void *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
 
 // Eight consecutive elements k0 .. k0+7 of a row of K elements, zeros at and past K, for rows whose
 // length is not a multiple of 8 (pieces straddle nothing, but the row may end inside one): element by
@@ -57,6 +80,9 @@ __device__ __forceinline__ u32x4 load8_slow(const uint16_t *row, int k0, int K) 
     }
     return u32x4{r0, r1, r2, r3};
 }
+
+// a * b + c for a, b below 2^24: one instruction
+__device__ __forceinline__ uint32_t mad24(uint32_t a, uint32_t b, uint32_t c) { return __umul24(a, b) + c; }
 
 // NK = 32-wide k steps (head dimension padded to 32 * NK).  VEC: the segment's K is a multiple of 8, its
 // rows come as 16-byte loads; otherwise element by element.  The two are separate instances of the whole
@@ -81,26 +107,42 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
 
     // A negative scale is applied as |scale| to negated scores (sign bits of the query operand flipped),
     // so that the running maximum is always the value to subtract.
+    // A scale of zero (uniform probabilities) is applied as scores of zero under a scale of one: the keys past
+    // the end of a segment are masked as -inf scores, which a zero factor would turn into NaN.
     const float c_signed = a.scale * kLog2e;
-    const float c = __builtin_fabsf(c_signed);
+    const float c = c_signed == 0.f ? 1.0f : __builtin_fabsf(c_signed);
     const uint32_t flip = c_signed < 0.f ? 0x80008000u : 0u;
+    const uint32_t keep = c_signed == 0.f ? 0u : 0xffffffffu;
     const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
 
-    // Staging, per thread: NK 16-byte pieces of the key rows (piece u = step * 256 + tid: row u / kPieces,
-    // column 8 * (u % kPieces)) and 4 keys x 8 columns of values (key group tid % 16, piece tid / 16; a load
+    // Staging, per thread: kSteps 16-byte pieces of the key rows (kLpr neighbouring lanes share a row; step s
+    // takes rows s * kRowsStep ..) and 4 keys x 8 columns of values (key group tid % 16, piece tid / 16; a load
     // instruction of a wavefront then covers 64 contiguous bytes of sixteen rows, a write 128 of one).  Element
     // offsets inside a segment fit 32 bits (checked by the kernel).
+    constexpr int kLpr = NK == 3 ? 16 : kPieces;      // lanes per key row (a power of two; 12 pieces: 4 lanes idle)
+    constexpr int kSteps = kLpr / 4, kRowsStep = kAttThreads / kLpr;
+    const int k_row = tid / kLpr, k_piece = tid % kLpr;
     const int v_kg = tid & 15, v_piece = tid >> 4;    // sixteen lanes = the sixteen key groups of one piece
     const bool v_thread = v_piece < kPieces;
-    uint32_t k_col[NK], k_off[NK];
-#pragma unroll
-    for (int step = 0; step < NK; ++step) {
-        const int u = step * kAttThreads + tid;
-        k_col[step] = (uint32_t)max(min(8 * (u % kPieces), K - 8), 0);
-        k_off[step] = (uint32_t)(u / kPieces) * (uint32_t)K + k_col[step];
-    }
-    const uint32_t v_col = (uint32_t)max(min(8 * v_piece, K - 8), 0);
-    const uint32_t v_off = (uint32_t)(4 * v_kg) * (uint32_t)K + v_col;
+    // Keys along an LDS row of transposed values stand in the order the probabilities have in a lane's registers:
+    // the eight keys 32 cc + 16 h + 4 rg + e (h < 2, e < 4) of lane group rg are 16 contiguous bytes, one operand
+    // read.  The thread's four keys 4 v_kg .. + 3 (v_kg = 8 cc + 4 h + rg) go to the 8-byte slot 8 cc + 2 rg + h.
+    const int v_slot = (v_kg & 8) + 2 * (v_kg & 3) + ((v_kg >> 2) & 1);
+    // VEC: the loads go through buffer descriptors that span exactly the segment's keys and values, so a row
+    // past the last key reads as zeros with no code; a piece past the head dimension has an offset that is
+    // out of range and stays there (its advance is multiplied by zero).
+    const __amdgpu_buffer_rsrc_t resK = __builtin_amdgcn_make_buffer_rsrc((void *)ks, 0, VEC ? N * K * 2 : 0, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t resV = __builtin_amdgcn_make_buffer_rsrc((void *)vs, 0, VEC ? N * K * 2 : 0, kRsrcFlags);
+    constexpr uint32_t kNever = 0xfffffff0u;
+    const uint32_t row_bytes = 2u * (uint32_t)K;      // all advances below are under 2^24 (K <= 128)
+    const uint32_t k_live = 8 * k_piece < K ? 1u : 0u, v_live = 8 * v_piece < K ? 1u : 0u;
+    const uint32_t k_byte0 = k_live ? (uint32_t)k_row * row_bytes + 16u * (uint32_t)k_piece : kNever;
+    const uint32_t v_byte0 = v_live ? (uint32_t)(4 * v_kg) * row_bytes + 16u * (uint32_t)v_piece : kNever;
+
+    // operand reads: lane (j, rg) reads 16 bytes of key row 16 t + j at k = 32 s + 8 rg, of value row (output
+    // column) 16 t + j at the lane group's eight keys of half cc
+    const uint32_t k_addr = lds_offset(sK) + (uint32_t)(j * kPitchK + rg * 16);
+    const uint32_t v_addr = lds_offset(sV) + (uint32_t)(j * kAttPitchV + rg * 16);
 
     constexpr int kRoundRows = kAttRows * QT;           // queries per workgroup round
     for (int round = zblock; (int64_t)round * kRoundRows < M; round += a.ride_slots ? (1 << 24) : a.tile_zdim) {
@@ -123,7 +165,8 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
 #pragma unroll
             for (int s = 0; s < NK; ++s) {
                 qf[q][s] = 32 * s + 8 * rg < K ? qf[q][s] : zero4;
-                qf[q][s] = u32x4{qf[q][s][0] ^ flip, qf[q][s][1] ^ flip, qf[q][s][2] ^ flip, qf[q][s][3] ^ flip};
+                qf[q][s] = u32x4{(qf[q][s][0] ^ flip) & keep, (qf[q][s][1] ^ flip) & keep, (qf[q][s][2] ^ flip) & keep,
+                                 (qf[q][s][3] ^ flip) & keep};
             }
         }
         float m[QT], lsum[QT];
@@ -139,49 +182,32 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
         // matrix work on block kb and land in registers (kw: this thread's pieces of the key rows, vw: its
         // 4 keys x 8 columns of values) while that work runs.  All loads of a block sit in one branch-free
         // sequence (index clamped, value selected afterwards): loads behind a branch wait one by one.
-        u32x4 kw[NK], vw[4];
-        auto fetch = [&](int kb) {
-            const bool full = kb + kAttKeys <= N;      // uniform: every row of the block exists
+        u32x4 kw[kSteps], vw[4];
+        uint32_t k_byte = k_byte0, v_byte = v_byte0;
+        auto fetch = [&](int kb) {                     // called for kb = 0, 64, 128, .. in turn
             if constexpr (VEC) {
-                if (full) {
-                    const uint32_t base = (uint32_t)kb * (uint32_t)K;
 #pragma unroll
-                    for (int step = 0; step < NK; ++step)
-                        kw[step] = *reinterpret_cast<const u32x4_unaligned *>(ks + (base + k_off[step]));
+                for (int step = 0; step < kSteps; ++step)
+                    kw[step] = __builtin_amdgcn_raw_buffer_load_b128(
+                        resK, mad24(k_live, (uint32_t)(step * kRowsStep) * row_bytes, k_byte), 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        vw[i] = *reinterpret_cast<const u32x4_unaligned *>(vs + (base + v_off + (uint32_t)(i * K)));
-                } else {
-#pragma unroll
-                    for (int step = 0; step < NK; ++step) {
-                        const int u = step * kAttThreads + tid;
-                        const uint32_t row = (uint32_t)min(kb + u / kPieces, N - 1);
-                        kw[step] = *reinterpret_cast<const u32x4_unaligned *>(ks + (row * (uint32_t)K + k_col[step]));
-                    }
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const uint32_t row = (uint32_t)min(kb + 4 * v_kg + i, N - 1);   // threads that do not store load a clamped row
-                        vw[i] = *reinterpret_cast<const u32x4_unaligned *>(vs + (row * (uint32_t)K + v_col));
-                    }
-                }
+                for (int i = 0; i < 4; ++i)
+                    vw[i] = __builtin_amdgcn_raw_buffer_load_b128(
+                        resV, mad24(v_live, (uint32_t)i * row_bytes, v_byte), 0, 0);
+                k_byte = mad24(k_live, (uint32_t)kAttKeys * row_bytes, k_byte);
+                v_byte = mad24(v_live, (uint32_t)kAttKeys * row_bytes, v_byte);
             } else {
 #pragma unroll
-                for (int step = 0; step < NK; ++step) {
-                    const int u = step * kAttThreads + tid;
-                    kw[step] = load8_slow(ks + (int64_t)min(kb + u / kPieces, N - 1) * K, 8 * (u % kPieces), K);
-                }
+                for (int step = 0; step < kSteps; ++step)
+                    kw[step] = load8_slow(ks + (int64_t)min(kb + step * kRowsStep + k_row, N - 1) * K, 8 * k_piece, K);
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     vw[i] = load8_slow(vs + (int64_t)min(kb + 4 * v_kg + i, N - 1) * K, 8 * v_piece, K);
-            }
-            // zeros past the head dimension and past the last key (values: their probabilities are zeros
-            // too, but 0 * stale bits could be NaN)
-            if (!full || K != KP) {
+                // zeros past the head dimension and past the last key (values: their probabilities are zeros
+                // too, but 0 * stale bits could be NaN)
 #pragma unroll
-                for (int step = 0; step < NK; ++step) {
-                    const int u = step * kAttThreads + tid;
-                    kw[step] = (kb + u / kPieces < N && 8 * (u % kPieces) < K) ? kw[step] : zero4;
-                }
+                for (int step = 0; step < kSteps; ++step)
+                    kw[step] = (kb + step * kRowsStep + k_row < N && 8 * k_piece < K) ? kw[step] : zero4;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) vw[i] = (kb + 4 * v_kg + i < N && 8 * v_piece < K) ? vw[i] : zero4;
             }
@@ -191,10 +217,10 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
         for (int kb = 0; kb < N; kb += kAttKeys) {
             __syncthreads();                           // the previous block (or round) is consumed
             // ---- keys: sK[key][k], one 16-byte piece per thread and step, pieces of a row on neighbouring lanes
+            if (kLpr == kPieces || k_piece < kPieces) {
 #pragma unroll
-            for (int step = 0; step < NK; ++step) {
-                const int u = step * kAttThreads + tid;
-                *reinterpret_cast<u32x4 *>(sK + (u / kPieces) * kPitchK + (u % kPieces) * 16) = kw[step];
+                for (int step = 0; step < kSteps; ++step)
+                    *reinterpret_cast<u32x4 *>(sK + (step * kRowsStep + k_row) * kPitchK + k_piece * 16) = kw[step];
             }
             // ---- values, transposed: 8 runs of 4 keys, one per column of the thread's piece
             if (v_thread) {
@@ -204,7 +230,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
                     const uint32_t lo23 = __builtin_amdgcn_perm(vw[3][w], vw[2][w], 0x05040100u);
                     const uint32_t hi01 = __builtin_amdgcn_perm(vw[1][w], vw[0][w], 0x07060302u);
                     const uint32_t hi23 = __builtin_amdgcn_perm(vw[3][w], vw[2][w], 0x07060302u);
-                    unsigned char *dst = sV + (8 * v_piece + 2 * w) * kAttPitchV + v_kg * 8;
+                    unsigned char *dst = sV + (8 * v_piece + 2 * w) * kAttPitchV + v_slot * 8;
                     *reinterpret_cast<u32x2 *>(dst) = u32x2{lo01, lo23};
                     *reinterpret_cast<u32x2 *>(dst + kAttPitchV) = u32x2{hi01, hi23};
                 }
@@ -222,15 +248,22 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
                 for (int q = 0; q < NQ; ++q)
     #pragma unroll
                     for (int t = 0; t < 4; ++t) sacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+                u32x4 ring[kAttRing];
+                {
+                    constexpr int kReads = 4 * NK;         // read i: k step i / 4, key tile i % 4
+                    static_for<kAttRing>([&](auto ic) {
+                        constexpr int I = decltype(ic)::value;
+                        if constexpr (I < kReads) lds_read128<16 * (I % 4) * kPitchK + 64 * (I / 4)>(ring[I], k_addr);
+                    });
+                    static_for<kReads>([&](auto ic) {
+                        constexpr int I = decltype(ic)::value, R = I % kAttRing;
+                        constexpr int kBehind = (I + kAttRing < kReads ? I + kAttRing : kReads) - (I + 1);
+                        lds_wait<kBehind>(ring[R]);
     #pragma unroll
-                for (int s = 0; s < NK; ++s) {
-    #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const u32x4 kf = *reinterpret_cast<const u32x4 *>(sK + (16 * t + j) * kPitchK + (4 * s + rg) * 16);
-    #pragma unroll
-                        for (int q = 0; q < NQ; ++q)
-                            sacc[q][t] = Elem<DT>::mfma(kf, qf[q][s], sacc[q][t]);
-                    }
+                        for (int q = 0; q < NQ; ++q) sacc[q][I % 4] = Elem<DT>::mfma(ring[R], qf[q][I / 4], sacc[q][I % 4]);
+                        if constexpr (I + kAttRing < kReads)
+                            lds_read128<16 * ((I + kAttRing) % 4) * kPitchK + 64 * ((I + kAttRing) / 4)>(ring[R], k_addr);
+                    });
                 }
                 // ---- online softmax; lane holds keys kb + 16 t + 4 rg + e of query j of each strip
                 const int left = N - kb;                   // keys of this block that exist
@@ -238,18 +271,24 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     f32x4(&sc)[4] = sacc[q];
-                    float bm = -INFINITY;
+                    // keys past the segment's last: -inf, so that they neither raise the maximum nor count
+                    // (their exponentials are zeros)
                     if (left < kAttKeys) {
     #pragma unroll
                         for (int t = 0; t < 4; ++t)
     #pragma unroll
                             for (int e = 0; e < 4; ++e) sc[t][e] = 16 * t + 4 * rg + e < left ? sc[t][e] : -INFINITY;
                     }
-    #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-    #pragma unroll
-                        for (int e = 0; e < 4; ++e) bm = fmaxf(bm, sc[t][e]);
-                    bm = quad_column_max(bm);
+                    settle_mfma(sc);                       // max3 reads the scores from inline assembly
+                    float bm;                              // one statement: no padding between its instructions
+                    asm volatile("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %0, %0, %6, %7\n\t"
+                                 "v_max3_f32 %0, %0, %8, %9\n\tv_max3_f32 %0, %0, %10, %11\n\tv_max3_f32 %0, %0, %12, %13\n\t"
+                                 "v_max3_f32 %0, %0, %14, %15\n\tv_max_f32 %0, %0, %16"
+                                 : "=&v"(bm)
+                                 : "v"(sc[0][0]), "v"(sc[0][1]), "v"(sc[0][2]), "v"(sc[0][3]), "v"(sc[1][0]), "v"(sc[1][1]),
+                                   "v"(sc[1][2]), "v"(sc[1][3]), "v"(sc[2][0]), "v"(sc[2][1]), "v"(sc[2][2]), "v"(sc[2][3]),
+                                   "v"(sc[3][0]), "v"(sc[3][1]), "v"(sc[3][2]), "v"(sc[3][3]));
+                    bm = quad_column_max_swap(bm);
                     // m is the reference the exponentials are taken against, not necessarily the maximum: it is
                     // raised (and the sums so far rescaled) only when a block's maximum passes it by more than
                     // 2^8 in the exponent, so probabilities stay below 256 (fine for both 16-bit types and the
@@ -267,7 +306,6 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             float p = __builtin_amdgcn_exp2f(fmaf(sc[t][e], c, bias));
-                            if (left < kAttKeys) p = 16 * t + 4 * rg + e < left ? p : 0.f;   // also when c = 0
                             sc[t][e] = p;
                             psum += p;
                         }
@@ -285,18 +323,22 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
                                           Elem<DT>::pack2(sc[2 * cc + 1][2], sc[2 * cc + 1][3])};
                 }
                 // ---- O^T += V^T P^T; a value operand read serves every strip
-    #pragma unroll
-                for (int cc = 0; cc < 2; ++cc) {
-    #pragma unroll
-                    for (int t = 0; t < kOutTiles; ++t) {
-                        const unsigned char *vrow = sV + (16 * t + j) * kAttPitchV + (32 * cc + 4 * rg) * 2;
-                        const u32x2 lo = *reinterpret_cast<const u32x2 *>(vrow);
-                        const u32x2 hi = *reinterpret_cast<const u32x2 *>(vrow + 32);
-                        const u32x4 vf = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                {
+                    constexpr int kReads = 2 * kOutTiles;  // read i: key half i / kOutTiles, output tile i % kOutTiles
+                    static_for<kAttRing>([&](auto ic) {
+                        constexpr int I = decltype(ic)::value;
+                        if constexpr (I < kReads) lds_read128<16 * (I % kOutTiles) * kAttPitchV + 64 * (I / kOutTiles)>(ring[I], v_addr);
+                    });
+                    static_for<kReads>([&](auto ic) {
+                        constexpr int I = decltype(ic)::value, R = I % kAttRing;
+                        constexpr int kBehind = (I + kAttRing < kReads ? I + kAttRing : kReads) - (I + 1);
+                        lds_wait<kBehind>(ring[R]);
     #pragma unroll
                         for (int q = 0; q < NQ; ++q)
-                            oacc[q][t] = Elem<DT>::mfma(vf, pf[q][cc], oacc[q][t]);
-                    }
+                            oacc[q][I % kOutTiles] = Elem<DT>::mfma(ring[R], pf[q][I / kOutTiles], oacc[q][I % kOutTiles]);
+                        if constexpr (I + kAttRing < kReads)
+                            lds_read128<16 * ((I + kAttRing) % kOutTiles) * kAttPitchV + 64 * ((I + kAttRing) / kOutTiles)>(ring[R], v_addr);
+                    });
                 }
             };
             if (QT == 1 || nq == 1) block_math(std::integral_constant<int, 1>{});

@@ -68,6 +68,16 @@ __device__ __forceinline__ float quad_column_max(float v) {
     v = fmaxf(v, __shfl_xor(v, 32));
     return v;
 }
+// The same through the two half-swaps of the register file (lanes 32.. of one register against lanes ..31 of
+// another, then odd rows of 16 against even rows): after each, the two registers hold both partners' values
+// in every lane.  No LDS round trip; the s_nop covers the distance a swap needs from the write of its operands.
+__device__ __forceinline__ float quad_column_max_swap(float v) {
+    float w;
+    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1\n\t"
+                 "v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1"
+                 : "+v"(v), "=&v"(w));
+    return v;
+}
 __device__ __forceinline__ float quad_column_sum(float v) {
     v += __shfl_xor(v, 16);
     v += __shfl_xor(v, 32);
