@@ -371,285 +371,11 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     }
 }
 
-// ---------------------------------------------------------------------------------------------------
-// The same pass for the common case K = 128 with 16-byte aligned key and value rows: keys and values go from
-// memory straight into LDS (no registers, no LDS write instructions), two buffers of 64 keys each, so that a
-// block costs one barrier and the loads of block b + 1 run under the arithmetic of block b.
-//   LDS row r of a buffer = key r of the block, 256 bytes, its sixteen 16-byte pieces permuted:
-//     keys:   piece p sits at position p ^ (r % 16); the operand read of lane (j, rg) for key 16 t + j,
-//             k = 32 s + 8 rg takes position (4 s + rg) ^ j -- sixteen lanes, sixteen positions, no conflict;
-//     values: piece p sits at position p ^ (2 (r % 4)).  The operand V^T (16 output columns x 32 keys) comes
-//             from transposing reads (ds_read_b64_tr_b16): in each group of sixteen lanes, lane 4 e + a points
-//             at four consecutive columns 16 t + 4 a .. of key row kappa_e, and lane i receives column
-//             16 t + i of kappa_0 .. kappa_3.  With kappa_e = 32 cc + 16 h + 4 rg + e these are the keys whose
-//             probabilities lane group rg holds in that order, so P still never moves between lanes.
-//   The row sums come from the matrix unit as well: a constant operand of ones in place of V^T adds up the
-//   rounded probabilities of each query over all 64 keys (one extra tile per key half).
-constexpr int kFastRow = 256, kFastBuf = kAttKeys * kFastRow;   // bytes per key row, per buffer
-
-template <int OFF> __device__ __forceinline__ void lds_read_tr(u32x2 &dst, uint32_t addr) {
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
-}
-template <int N> __device__ __forceinline__ void lds_wait2(u32x2 &x, u32x2 &y) {
-    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N) : "memory");
-}
-// Keeps the matrix instructions that produced acc above the statements that follow (the compiler would
-// otherwise collect them behind the reads of later steps and need registers for all those reads at once).
-__device__ __forceinline__ void pin(f32x4 &acc) { asm volatile("" : "+v"(acc)); }
-// 64 lanes x 16 bytes from base + off + OFF (per lane) to LDS at dst + OFF + 16 * lane
-template <int OFF> __device__ __forceinline__ void load_to_lds_at(uint32_t off, const void *base, uint32_t dst) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3" ::"v"(off), "s"(base), "s"(dst), "n"(OFF)
-                 : "memory", "m0");
-}
-__device__ __forceinline__ void load_to_lds(uint32_t off, const void *base, uint32_t dst) { load_to_lds_at<0>(off, base, dst); }
-
-template <int DT, int QT>
-__device__ __forceinline__ void attention_fast(const RunArgs &a, const void *Vbuf, const SegRec &rec, int64_t h, int zblock,
-                                               unsigned char *lds) {
-    constexpr int NK = 4, kOutTiles = 8;
-    const int M = rec.M, N = rec.N;
-    constexpr int K = 128;
-    const int tid = threadIdx.x;
-    const int wave = uniform(tid >> 6);
-    const int lane = lane_id();
-    const int j = lane & 15, rg = lane >> 4;
-    const uint16_t *qs = reinterpret_cast<const uint16_t *>(a.A) + h * a.Dm1 + rec.off1;
-    const unsigned char *ks = reinterpret_cast<const unsigned char *>(reinterpret_cast<const uint16_t *>(a.B) + h * a.Dm2 + rec.off2);
-    const unsigned char *vs = reinterpret_cast<const unsigned char *>(reinterpret_cast<const uint16_t *>(Vbuf) + h * a.Dm2 + rec.off2);
-    uint16_t *os = reinterpret_cast<uint16_t *>(a.out) + h * a.Dm1 + rec.off1;
-
-    const float c_signed = a.scale * kLog2e;           // see attention_body for the sign and the zero scale
-    const float c = c_signed == 0.f ? 1.0f : __builtin_fabsf(c_signed);
-    const uint32_t flip = c_signed < 0.f ? 0x80008000u : 0u;
-    const uint32_t keep = c_signed == 0.f ? 0u : 0xffffffffu;
-    const uint32_t one2 = DT == 0 ? 0x3c003c00u : 0x3f803f80u;
-    const u32x4 ones = u32x4{one2, one2, one2, one2};
-
-    // loads: instruction i of a wavefront fills LDS rows 16 wave + 4 i + lane / 16, position lane % 16.  The
-    // instruction's offset field moves the memory address and the LDS address alike, so instruction i is
-    // instruction 0 plus 4 i rows -- except for the permutation of the pieces: values, row modulo 4 = lane / 16 for
-    // every i; keys, (4 i + lane / 16) = an exclusive-or of 64 i on the byte position.
-    const uint32_t lds0 = lds_offset(lds);
-    const uint32_t ld_row = (uint32_t)(16 * wave + rg);
-    const uint32_t k_ld = ld_row * kFastRow + 16u * (uint32_t)(j ^ rg);
-    const uint32_t v_ld = ld_row * kFastRow + 16u * ((uint32_t)j ^ ((uint32_t)rg << 1));
-    // One load instruction of the block of keys kb .. kb + 63 into buffer buf: I < 4 keys, else values.  The
-    // texture path takes a while over 64 x 16 bytes; a wavefront that issues all eight at once waits for the
-    // other wavefronts' loads as well, so the full blocks' loads go out one by one between the matrix steps.
-    auto issue_one = [&](auto ic, int kb, int buf) {
-        constexpr int I = decltype(ic)::value, R = 4 * (I & 3) * kFastRow;
-        const uint32_t dk = lds0 + (uint32_t)(buf * kFastBuf + 16 * wave * kFastRow);
-        if constexpr (I < 4) load_to_lds_at<R>(k_ld ^ (uint32_t)(64 * I), ks + (int64_t)kb * kFastRow, dk);
-        else load_to_lds_at<R>(v_ld, vs + (int64_t)kb * kFastRow, dk + 2 * kFastBuf);
-    };
-    auto issue = [&](int kb, int buf) {                // all eight, also of a last block that is not full
-        const unsigned char *kbase = ks + (int64_t)kb * kFastRow, *vbase = vs + (int64_t)kb * kFastRow;
-        const uint32_t dk = lds0 + (uint32_t)(buf * kFastBuf + 16 * wave * kFastRow), dv = dk + 2 * kFastBuf;
-        const int last = N - 1 - kb;                   // rows past the last key repeat it (finite; masked below)
-        if (last >= kAttKeys - 1) {
-            static_for<8>([&](auto ic) { issue_one(ic, kb, buf); });
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                load_to_lds(min(ld_row + 4u * i, (uint32_t)last) * kFastRow + ((k_ld ^ (uint32_t)(64 * i)) & 255u), kbase,
-                            dk + (uint32_t)(4 * i * kFastRow));
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                load_to_lds(min(ld_row + 4u * i, (uint32_t)last) * kFastRow + (v_ld & 255u), vbase, dv + (uint32_t)(4 * i * kFastRow));
-        }
-    };
-    // operand reads (buffer 0): keys, per k step s; values, per output tile t % 4 (t / 4 and the key half are
-    // instruction offsets)
-    uint32_t k_rd[NK], v_rd[4];
-#pragma unroll
-    for (int s = 0; s < NK; ++s) k_rd[s] = lds0 + (uint32_t)(j * kFastRow + 16 * ((4 * s + rg) ^ j));
-    {
-        const int e = j >> 2, a4 = j & 3;
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-            v_rd[v] = lds0 + (uint32_t)(2 * kFastBuf + (4 * rg + e) * kFastRow + 16 * ((2 * v + (a4 >> 1)) ^ (2 * e)) + 8 * (a4 & 1));
-    }
-
-    constexpr int kRoundRows = kAttRows * QT;
-    int buf = 0;                                       // the buffer the operand reads point at
-    for (int round = zblock; (int64_t)round * kRoundRows < M; round += a.ride_slots ? (1 << 24) : a.tile_zdim) {
-        const int r0 = round * kRoundRows + wave * 16;
-        const int nq = uniform(r0 >= M ? 0 : min(QT, (M - r0 + kAttRows - 1) / kAttRows));
-        issue(0, buf);
-        u32x4 qf[QT][NK];
-#pragma unroll
-        for (int q = 0; q < QT; ++q) {
-            const uint16_t *qrow = qs + (int64_t)min(r0 + kAttRows * q + j, M - 1) * K;
-#pragma unroll
-            for (int s = 0; s < NK; ++s) {
-                const u32x4 x = *reinterpret_cast<const u32x4_unaligned *>(qrow + 32 * s + 8 * rg);
-                qf[q][s] = u32x4{(x[0] ^ flip) & keep, (x[1] ^ flip) & keep, (x[2] ^ flip) & keep, (x[3] ^ flip) & keep};
-            }
-        }
-        float m[QT];
-        f32x4 oacc[QT][kOutTiles], lacc[QT];
-#pragma unroll
-        for (int q = 0; q < QT; ++q) {
-            m[q] = -INFINITY;
-            lacc[q] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int t = 0; t < kOutTiles; ++t) oacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-
-        for (int kb = 0; kb < N; kb += kAttKeys, buf ^= 1) {
-            // the next block's loads: between the matrix steps below when it is a full block and this wavefront
-            // has queries, else all at once
-            const bool spread = false;
-            if (!spread && kb + kAttKeys < N) issue(kb + kAttKeys, buf ^ 1);
-            auto block_math = [&](auto nq_tag) {
-                constexpr int NQ = decltype(nq_tag)::value;
-                f32x4 sacc[NQ][4];
-    #pragma unroll
-                for (int q = 0; q < NQ; ++q)
-    #pragma unroll
-                    for (int t = 0; t < 4; ++t) sacc[q][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-                {
-                    u32x4 ring[kAttRing];
-                    constexpr int kReads = 4 * NK;         // read i: k step i / 4, key tile i % 4
-                    static_for<kAttRing>([&](auto ic) {
-                        constexpr int I = decltype(ic)::value;
-                        if constexpr (I < kReads) lds_read128<16 * (I % 4) * kFastRow>(ring[I], k_rd[I / 4]);
-                    });
-                    static_for<kReads>([&](auto ic) {
-                        constexpr int I = decltype(ic)::value, R = I % kAttRing;
-                        constexpr int kBehind = (I + kAttRing < kReads ? I + kAttRing : kReads) - (I + 1);
-                        lds_wait<kBehind>(ring[R]);
-    #pragma unroll
-                        for (int q = 0; q < NQ; ++q) {
-                            sacc[q][I % 4] = Elem<DT>::mfma(ring[R], qf[q][I / 4], sacc[q][I % 4]);
-                            pin(sacc[q][I % 4]);
-                        }
-                        if constexpr (I + kAttRing < kReads)
-                            lds_read128<16 * ((I + kAttRing) % 4) * kFastRow>(ring[R], k_rd[(I + kAttRing) / 4]);
-                        if constexpr (I % 4 == 1) {
-                            if (spread) issue_one(std::integral_constant<int, I / 4>{}, kb + kAttKeys, buf ^ 1);
-                        }
-                    });
-                }
-                // ---- online softmax; lane holds keys kb + 16 t + 4 rg + e of query j of each strip
-                const int left = N - kb;
-                u32x4 pf[NQ][2];
-    #pragma unroll
-                for (int q = 0; q < NQ; ++q) {
-                    f32x4(&sc)[4] = sacc[q];
-                    if (left < kAttKeys) {
-    #pragma unroll
-                        for (int t = 0; t < 4; ++t)
-    #pragma unroll
-                            for (int e = 0; e < 4; ++e) sc[t][e] = 16 * t + 4 * rg + e < left ? sc[t][e] : -INFINITY;
-                    }
-                    settle_mfma(sc);
-                    float bm;
-                    asm volatile("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %0, %0, %6, %7\n\t"
-                                 "v_max3_f32 %0, %0, %8, %9\n\tv_max3_f32 %0, %0, %10, %11\n\tv_max3_f32 %0, %0, %12, %13\n\t"
-                                 "v_max3_f32 %0, %0, %14, %15\n\tv_max_f32 %0, %0, %16"
-                                 : "=&v"(bm)
-                                 : "v"(sc[0][0]), "v"(sc[0][1]), "v"(sc[0][2]), "v"(sc[0][3]), "v"(sc[1][0]), "v"(sc[1][1]),
-                                   "v"(sc[1][2]), "v"(sc[1][3]), "v"(sc[2][0]), "v"(sc[2][1]), "v"(sc[2][2]), "v"(sc[2][3]),
-                                   "v"(sc[3][0]), "v"(sc[3][1]), "v"(sc[3][2]), "v"(sc[3][3]));
-                    bm = quad_column_max_swap(bm);
-                    const bool raise = !((bm - m[q]) * c <= 8.0f);   // see attention_body
-                    const float m_new = raise ? bm : m[q];
-                    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                    const float alpha = !raise ? 1.0f : m[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m[q] - m_use) * c);
-                    m[q] = m_new;
-                    const float bias = -m_use * c;
-    #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-    #pragma unroll
-                        for (int e = 0; e < 4; ++e) sc[t][e] = __builtin_amdgcn_exp2f(fmaf(sc[t][e], c, bias));
-                    if (__any(raise)) {
-                        lacc[q] *= alpha;
-    #pragma unroll
-                        for (int t = 0; t < kOutTiles; ++t) oacc[q][t] *= alpha;
-                    }
-    #pragma unroll
-                    for (int cc = 0; cc < 2; ++cc)
-                        pf[q][cc] = u32x4{Elem<DT>::pack2(sc[2 * cc][0], sc[2 * cc][1]), Elem<DT>::pack2(sc[2 * cc][2], sc[2 * cc][3]),
-                                          Elem<DT>::pack2(sc[2 * cc + 1][0], sc[2 * cc + 1][1]),
-                                          Elem<DT>::pack2(sc[2 * cc + 1][2], sc[2 * cc + 1][3])};
-                }
-                // ---- O^T += V^T P^T and the row sums
-                {
-                    u32x2 lo[kAttRing], hi[kAttRing];
-                    constexpr int kReads = 2 * kOutTiles;  // step i: key half i / kOutTiles, output tile i % kOutTiles
-                    static_for<kAttRing>([&](auto ic) {
-                        constexpr int I = decltype(ic)::value, T = I % kOutTiles, CC = I / kOutTiles;
-                        lds_read_tr<32 * CC * kFastRow + 128 * (T / 4)>(lo[I], v_rd[T % 4]);
-                        lds_read_tr<(32 * CC + 16) * kFastRow + 128 * (T / 4)>(hi[I], v_rd[T % 4]);
-                    });
-    #pragma unroll
-                    for (int q = 0; q < NQ; ++q)
-    #pragma unroll
-                        for (int cc = 0; cc < 2; ++cc) lacc[q] = Elem<DT>::mfma(ones, pf[q][cc], lacc[q]);
-                    static_for<kReads>([&](auto ic) {
-                        constexpr int I = decltype(ic)::value, R = I % kAttRing;
-                        constexpr int kBehind = (I + kAttRing < kReads ? I + kAttRing : kReads) - (I + 1);
-                        lds_wait2<2 * kBehind>(lo[R], hi[R]);
-                        const u32x4 vf = u32x4{lo[R][0], lo[R][1], hi[R][0], hi[R][1]};
-    #pragma unroll
-                        for (int q = 0; q < NQ; ++q) {
-                            oacc[q][I % kOutTiles] = Elem<DT>::mfma(vf, pf[q][I / kOutTiles], oacc[q][I % kOutTiles]);
-                            pin(oacc[q][I % kOutTiles]);
-                        }
-                        if constexpr (I + kAttRing < kReads) {
-                            constexpr int J = I + kAttRing, T = J % kOutTiles, CC = J / kOutTiles;
-                            lds_read_tr<32 * CC * kFastRow + 128 * (T / 4)>(lo[R], v_rd[T % 4]);
-                            lds_read_tr<(32 * CC + 16) * kFastRow + 128 * (T / 4)>(hi[R], v_rd[T % 4]);
-                        }
-                        if constexpr (I % 4 == 1) {
-                            if (spread) issue_one(std::integral_constant<int, 4 + I / 4>{}, kb + kAttKeys, buf ^ 1);
-                        }
-                    });
-                }
-            };
-            if (nq > 0) {
-                if (QT == 1 || nq == 1) block_math(std::integral_constant<int, 1>{});
-                else block_math(std::integral_constant<int, QT>{});
-            }
-            {                                                  // the operand reads move to the other buffer
-                const uint32_t step = buf ? (uint32_t)-kFastBuf : (uint32_t)kFastBuf;
-#pragma unroll
-                for (int s = 0; s < NK; ++s) k_rd[s] += step;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) v_rd[v] += step;
-            }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's part of the next block is in LDS
-            __syncthreads();                                   // .. and everybody's; this block's buffer is free
-        }
-        // ---- normalise and store: lane (query j, rg) holds columns 16 t + 4 rg + e; every element of lacc is
-        // the query's row sum
-#pragma unroll
-        for (int q = 0; q < QT; ++q) {
-            if (q >= nq) continue;
-            const int qr = r0 + kAttRows * q + j;
-            const float inv = 1.0f / lacc[q][0];
-            if (qr < M) {
-                uint16_t *orow = os + (int64_t)qr * K;
-#pragma unroll
-                for (int t = 0; t < kOutTiles; ++t)
-                    *reinterpret_cast<u32x2_unaligned *>(orow + 16 * t + 4 * rg) =
-                        u32x2{Elem<DT>::pack2(oacc[q][t][0] * inv, oacc[q][t][1] * inv),
-                              Elem<DT>::pack2(oacc[q][t][2] * inv, oacc[q][t][3] * inv)};
-            }
-        }
-    }
-}
-
 template <int DT, int NK, int QT>
 __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
     constexpr int KP = 32 * NK;
-    constexpr bool kHasFast = NK == 4 && QT == 2;     // the instance that takes K = 128 straight into LDS
-    constexpr int kBytesK = kAttKeys * (KP * 2 + 16), kBytesV = KP * kAttPitchV;
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[kHasFast ? 4 * kFastBuf : kBytesK + kBytesV];
-    unsigned char *sK = smem, *sV = smem + kBytesK;
+    __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 16)];
+    __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
     if (!header_ok(a)) { report_mismatch(a); return; }
     // Workgroup -> (segment, head, row block).  Consecutive workgroup ids go to the eight dies of the chip in
     // turn, and each die has its own L2: id = die + 8 k.  All row blocks of one (segment, head) pair read the
@@ -693,15 +419,6 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void at
         if (h == 0 && zblock == 0 && threadIdx.x == 0)
             atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
-    }
-    if constexpr (kHasFast) {
-        // K = 128, at least one key, key and value rows on 16-byte boundaries: straight into LDS
-        const uintptr_t kbits = (uintptr_t)(reinterpret_cast<const uint16_t *>(a.B) + h * a.Dm2 + rec.off2);
-        const uintptr_t vbits = (uintptr_t)(reinterpret_cast<const uint16_t *>(Vbuf) + h * a.Dm2 + rec.off2);
-        if (K == 128 && rec.N > 0 && ((kbits | vbits) & 15) == 0) {
-            attention_fast<DT, QT>(a, Vbuf, rec, h, zblock, smem);
-            return;
-        }
     }
     if ((K & 7) == 0) attention_body<DT, NK, QT, true>(a, Vbuf, rec, h, zblock, sK, sV);
     else attention_body<DT, NK, QT, false>(a, Vbuf, rec, h, zblock, sK, sV);
