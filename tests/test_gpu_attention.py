@@ -71,6 +71,14 @@ def test_head_dimensions_not_multiples_of_eight_and_odd_offsets(dev):
     run(dev, M, N, K, 1, torch.bfloat16, 0.1, seed=2)
 
 
+def test_vector_loads_at_odd_element_offsets(dev):
+    # segments whose head dimension is a multiple of 8 (16-byte loads through the segment's buffer descriptor)
+    # but that start at an odd element: the segments before them have odd sizes
+    M = [3, 40, 5, 70, 1, 130]; N = [5, 100, 7, 65, 3, 200]; K = [5, 64, 7, 128, 1, 96]
+    run(dev, M, N, K, 2, torch.float16, 0.2, seed=5)
+    run(dev, M, N, K, 3, torch.bfloat16, 0.1, seed=6)
+
+
 def test_empty_segments_and_no_keys(dev):
     # M = 0: nothing; N = 0: zeros (a sum over no keys)
     M = [4, 0, 9, 30]; N = [6, 5, 0, 70]; K = [16, 8, 24, 64]
@@ -94,6 +102,10 @@ def test_negative_and_zero_scale(dev):
     M = [9, 70]; N = [100, 17]; K = [16, 64]
     for scale in (-0.3, 0.0):
         run(dev, M, N, K, 2, torch.float16, scale)
+    # tall segments (two strips per wavefront), last key block ragged: a zero scale must still give the mean of
+    # the values over the keys that exist
+    for scale in (-0.2, 0.0):
+        run(dev, [300, 520], [130, 77], [128, 64], 2, torch.bfloat16, scale, seed=7)
 
 
 def test_long_segments_many_key_blocks(dev):
