@@ -38,9 +38,12 @@ constexpr int kAttWaves = kAttThreads / 64;
 constexpr int kAttKeys = 64;                          // keys per block
 constexpr int kAttRows = 16 * kAttWaves;              // queries per workgroup round
 static_assert(kAttRows == kAttBlockRows, "the plan's row-block prefixes count blocks of kAttRows and 2 kAttRows");
-constexpr int kAttPitchV = kAttKeys * 2 + 16;         // bytes per LDS row of transposed values: the sixteen rows
-// 16 t + j that an operand read (16 bytes per lane) touches start in sixteen different groups of four banks, and
-// a staging write (8 bytes per lane, 32 lanes at a time) covers two rows that lie 32 banks apart.
+// LDS row pitches.  A 16-byte operand read of a wavefront is served 32 lanes at a time, 512 bytes wide (measured:
+// lane * 16 and 288-byte rows run at 4.75 cycles per wavefront read, 272- and 144-byte rows at 8): the lanes
+// (j, rg) and (j, rg + 1) of sixteen rows j must land in 32 different 16-byte slots modulo 512 bytes, which a
+// pitch of 16 * (2 * odd) bytes does.  Keys: 64 NK + 32 bytes; transposed values (64 keys a row): 160 bytes.  The
+// staging writes take what is left (two-way conflicts on a quarter as many instructions).
+constexpr int kAttPitchV = kAttKeys * 2 + 32;
 constexpr int kAttRing = 6;                           // LDS operand reads in flight per wavefront
 
 // LDS operand reads as inline assembly, so that kAttRing of them are in flight under the matrix instructions
@@ -91,8 +94,7 @@ template <int DT, int NK, int QT, bool VEC>
 __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbuf, const SegRec &rec, int64_t h, int zblock,
                                                unsigned char *sK, unsigned char *sV) {
     constexpr int KP = 32 * NK;                       // padded head dimension
-    constexpr int kPitchK = KP * 2 + 16;              // bytes per LDS row of keys (16-byte skew: 16 lanes of
-                                                      // a 16-byte read cover all banks once)
+    constexpr int kPitchK = KP * 2 + 32;              // bytes per LDS row of keys
     constexpr int kPieces = KP / 8;                   // 16-byte pieces per row
     constexpr int kOutTiles = KP / 16;
     const int M = rec.M, N = rec.N, K = rec.K;
@@ -374,7 +376,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
 template <int DT, int NK, int QT>
 __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
     constexpr int KP = 32 * NK;
-    __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 16)];
+    __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 32)];
     __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
     if (!header_ok(a)) { report_mismatch(a); return; }
     // Workgroup -> (segment, head, row block).  Consecutive workgroup ids go to the eight dies of the chip in
