@@ -416,8 +416,9 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void at
     const SegRec rec = load_rec(pv.recs, g);
     const int M = rec.M, K = rec.K;
     if (M < 1 || K < 1) return;
-    // the launch was sized for a smaller head dimension, or element offsets inside the segment pass 32 bits
-    if (K > KP || (int64_t)max(M, rec.N) * K >= (int64_t(1) << 31)) {
+    // the launch was sized for a smaller head dimension, or byte offsets inside the segment (of a last block of
+    // keys that reaches past the segment's end, too) pass 32 bits
+    if (K > KP || ((int64_t)max(M, rec.N) + kAttKeys) * K >= (int64_t(1) << 31)) {
         if (h == 0 && zblock == 0 && threadIdx.x == 0)
             atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
