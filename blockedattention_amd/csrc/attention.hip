@@ -44,7 +44,10 @@ static_assert(kAttRows == kAttBlockRows, "the plan's row-block prefixes count bl
 // pitch of 16 * (2 * odd) bytes does.  Keys: 64 NK + 32 bytes; transposed values (64 keys a row): 160 bytes.  The
 // staging writes take what is left (two-way conflicts on a quarter as many instructions).
 constexpr int kAttPitchV = kAttKeys * 2 + 32;
-constexpr int kAttRing = 6;                           // LDS operand reads in flight per wavefront
+// LDS operand reads in flight per wavefront: six, or three in the builds for short segments and head dimensions
+// up to 64, which then fit 128 registers and run four wavefronts per SIMD (the launch is bound by the life of a
+// workgroup there: 256 segments of 32..128 rows, 31.3 -> 29.0 us)
+constexpr int att_ring(int nk, int qt) { return qt == 1 && nk <= 2 ? 3 : 6; }
 
 // LDS operand reads as inline assembly, so that kAttRing of them are in flight under the matrix instructions
 // (left to itself the compiler, short of registers, issues each read right before its use and every matrix
@@ -97,6 +100,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
     constexpr int kPitchK = KP * 2 + 32;              // bytes per LDS row of keys
     constexpr int kPieces = KP / 8;                   // 16-byte pieces per row
     constexpr int kOutTiles = KP / 16;
+    constexpr int kAttRing = att_ring(NK, QT);
     const int M = rec.M, N = rec.N, K = rec.K;
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
@@ -374,7 +378,7 @@ __device__ __forceinline__ void attention_body(const RunArgs &a, const void *Vbu
 }
 
 template <int DT, int NK, int QT>
-__global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 1 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
+__global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 2 ? 4 : 3) void attention_kernel(RunArgs a, const void *Vbuf) {
     constexpr int KP = 32 * NK;
     __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 32)];
     __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
@@ -453,7 +457,7 @@ int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg
         nseg = info->nseg;
         nk = std::max(1, (info->max_K + 31) / 32);
         max_m = std::max<int64_t>(info->max_M, 1);
-        if (info->total_rows >= 128 * std::max<int64_t>(nseg, 1)) qt = 2;   // mean segment height >= 128
+        if (info->total_rows >= 256 * std::max<int64_t>(nseg, 1)) qt = 2;   // mean segment height >= 256 (136: one strip is 6 % faster)
     }
     if (forced == 1 || forced == 2) qt = forced;
     // Row blocks per pair: enough for the tallest segment, but no more than four times what the mean segment
