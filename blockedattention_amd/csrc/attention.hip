@@ -382,6 +382,8 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 2 ? 4 : 3) void at
     constexpr int KP = 32 * NK;
     __shared__ __attribute__((aligned(16))) unsigned char sK[kAttKeys * (KP * 2 + 32)];
     __shared__ __attribute__((aligned(16))) unsigned char sV[KP * kAttPitchV];
+    // (the row blocks per head come with the header: one memory round trip less than the prefix's last entry)
+    const int64_t per_head = QT == 2 ? ((ConstHdr)(uintptr_t)a.plan)->att_blocks128 : ((ConstHdr)(uintptr_t)a.plan)->att_blocks64;
     if (!header_ok(a)) { report_mismatch(a); return; }
     // Workgroup -> (segment, head, row block).  Consecutive workgroup ids go to the eight dies of the chip in
     // turn, and each die has its own L2: id = die + 8 k.  All row blocks of one (segment, head) pair read the
@@ -397,7 +399,6 @@ __global__ __launch_bounds__(kAttThreads, QT == 2 ? 2 : NK <= 2 ? 4 : 3) void at
     int64_t h;
     if (a.ride_slots) {
         const int32_t *pfx = plan_rowblocks(a.plan, a.nseg, QT - 1);
-        const int64_t per_head = ((ConstI32)(uintptr_t)pfx)[a.nseg];
         const int64_t items = per_head * a.H, share = (items + 7) >> 3;
         const int64_t u = (int64_t)die * share + kk;
         // a grid too small for the plan's items: the host summary the launch was sized from is not this plan's

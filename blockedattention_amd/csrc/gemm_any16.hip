@@ -82,6 +82,7 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char sY[kAnyTile * kAnyPitch];
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
     const int nseg = hdr->nseg;
+    const int64_t per_head = hdr->att_blocks64;       // 64-row rounds per head (= the row-block prefix's last entry)
     if (!header_ok(a)) {
         report_mismatch(a);
         return;
@@ -96,7 +97,6 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
     int64_t h;
     if (a.ride_slots) {
         const int32_t *pfx = plan_rowblocks(a.plan, nseg, 0);
-        const int64_t per_head = ((ConstI32)(uintptr_t)pfx)[nseg];
         const int64_t u = blockIdx.x;
         if (u >= per_head * a.H) return;
         h = u % a.H;                                   // consecutive workgroups: the heads of one round, one shape
