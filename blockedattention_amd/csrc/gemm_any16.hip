@@ -5,10 +5,11 @@
 // reduces over N, dB = dS^T A over M, with dS and the saved operands read as they lie).
 //
 // Workgroup = 64 rows x 64 columns of one segment and head at a time, k in chunks of 64.  Both operand chunks go
-// through LDS as [row][k] (k contiguous, row pitch 144 bytes: the sixteen rows a quarter-wavefront reads together
-// start in sixteen different bank groups).  Staging reads 16 bytes per lane along whatever dimension is contiguous
+// through LDS with a row pitch of 160 bytes.  Staging reads 16 bytes per lane along whatever dimension is contiguous
 // in memory, at any 2-byte alignment, through a buffer descriptor that spans exactly the segment (rows past its
-// end read as zeros); an operand stored k-major is transposed on the way in (2-byte LDS writes).  Each wavefront
+// end read as zeros), and writes them to LDS as they come: an operand that is not transposed lies there as
+// [row][k] and is read 16 bytes per lane; an operand stored k-major lies there k-major and the matrix operand is
+// gathered by the transposing LDS read (ds_read_b64_tr_b16, four k of one row per lane).  Each wavefront
 // then computes 16 rows x 64 columns as four 16 x 16 tiles with v_mfma_f32_16x16x32 (fp32 sums).  Column slot n of
 // tile t is column 4 n + t, so a lane owns four consecutive columns of each of its rows and the sixteen lanes of a
 // row group write 128 contiguous bytes.
@@ -21,7 +22,8 @@ namespace ba {
 constexpr int kAnyThreads = 256;
 constexpr int kAnyWaves = kAnyThreads / 64;
 constexpr int kAnyTile = 64;                         // rows and columns per workgroup step, k per chunk
-constexpr int kAnyPitch = (kAnyTile + 8) * 2;        // bytes per LDS row
+constexpr int kAnyPitch = (kAnyTile + 16) * 2;       // bytes per LDS row: 160 = 16 * (2 * odd), the pitch at which the
+// 16-byte operand reads (served 32 lanes, 512 bytes at a time) and the transposing 8-byte reads meet no bank conflict
 
 // Sixteen consecutive elements of the segment from byte offset `off` on (kNoLine: zeros).  Two 16-byte loads where
 // they lie inside the segment; a piece that reaches past its end is fetched element by element, the hardware
@@ -58,22 +60,43 @@ __device__ __forceinline__ Line16 fetch_chunk16(__amdgpu_buffer_rsrc_t res, bool
     const int lead = transposed ? k * rows + row : row * K + k;
     return load_line16(res, row < rows && k < K ? (uint32_t)lead * 2u : kNoLine, bytes);
 }
+// Into LDS.  An operand that is not transposed lies as dst[row][k].  A transposed one stays k-major, dst[k][..], and
+// the matrix operand is gathered by transposing reads (lds_tr8 below): 16-byte writes here instead of sixteen 2-byte
+// ones.  X (rows of the output) keeps its rows in order.  Y (columns of the output) permutes each group of sixteen
+// columns, 16 a + 4 b + t -> position 16 t + 4 a + b, so that the lane that reads position 16 t + i of a row gets
+// column 4 i + t: the columns a lane stores side by side (see the kernel).
+template <bool PERMUTE>
 __device__ __forceinline__ void put_chunk16(Line16 x, bool transposed, int rows, int K, int r0, int k0, unsigned char *dst,
                                             int tid) {
     const int line = tid >> 2, part = (tid & 3) * 16;
-    if (!transposed) {
-        const int valid = K - (k0 + part);           // elements of the row from here on; the rest belongs to the next row
+    const int valid = transposed ? rows - (r0 + part) : K - (k0 + part);   // elements of the line from here on
 #pragma unroll
-        for (int i = 0; i < 16; ++i) x.e[i] = i < valid ? x.e[i] : (uint16_t)0;
+    for (int i = 0; i < 16; ++i) x.e[i] = i < valid ? x.e[i] : (uint16_t)0;
+    if (!PERMUTE || !transposed) {
         u32x4 *d = reinterpret_cast<u32x4 *>(dst + line * kAnyPitch + part * 2);
         d[0] = x.v[0];
         d[1] = x.v[1];
     } else {
-        const int valid = rows - (r0 + part);
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(&x);
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-            *reinterpret_cast<uint16_t *>(dst + (part + i) * kAnyPitch + line * 2) = i < valid ? x.e[i] : (uint16_t)0;
+        for (int t = 0; t < 4; ++t) {                 // elements t, 4 + t, 8 + t, 12 + t of the thread's sixteen
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+            const uint32_t lo = __builtin_amdgcn_perm(w[2 + (t >> 1)], w[t >> 1], sel);
+            const uint32_t hi = __builtin_amdgcn_perm(w[6 + (t >> 1)], w[4 + (t >> 1)], sel);
+            *reinterpret_cast<u32x2 *>(dst + line * kAnyPitch + 32 * t + (part >> 2) * 2) = u32x2{lo, hi};
+        }
     }
+}
+// Eight k of one row (column) of a k-major chunk as matrix operand: two transposing reads of four k each.  In a
+// group of sixteen lanes, lane 4 e + a points at positions 4 a .. 4 a + 3 of k row e, and lane i receives position
+// i of the four k rows; p is this lane's address for the first four k, the next four lie four rows on.
+__device__ __forceinline__ u32x4 lds_tr8(const unsigned char *p) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 *LdsPtr;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(uintptr_t)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(uintptr_t)(p + 4 * kAnyPitch));
+    const u32x2 l = __builtin_bit_cast(u32x2, lo), h = __builtin_bit_cast(u32x2, hi);
+    return u32x4{l[0], l[1], h[0], h[1]};
 }
 
 template <int DT>
@@ -129,6 +152,10 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
     // row 4 n + t of Y (column slot n of tile t is column 4 n + t), eight k from 8 q on
     const unsigned char *xa = sX + (16 * wave + n) * kAnyPitch + q * 16;
     const unsigned char *ya = sY + (4 * n) * kAnyPitch + q * 16;
+    // the same from k-major chunks (transposed operands): k row 8 q + n / 4 of the step, positions 4 (n % 4) .. of the
+    // wavefront's sixteen rows (X) or of tile t's sixteen positions (Y, + 32 t bytes)
+    const unsigned char *xt = sX + (8 * q + (n >> 2)) * kAnyPitch + (16 * wave + 4 * (n & 3)) * 2;
+    const unsigned char *yt = sY + (8 * q + (n >> 2)) * kAnyPitch + (4 * (n & 3)) * 2;
 
     // lane (n, q): rows 16 wave + 4 q + i, columns 64 cb + 4 n .. + 3; clears the accumulators for the next block
     auto store_block = [&](int cb, int r0, f32x4 (&acc)[4]) {
@@ -167,8 +194,8 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
         int cb = 0, kc = 0;
         for (int step = 0; step < steps; ++step) {
             __syncthreads();                                           // the previous chunk is consumed
-            put_chunk16(nx, t1, M, K, r0, kc * kAnyTile, sX, tid);
-            put_chunk16(ny, t2, N, K, cb * kAnyTile, kc * kAnyTile, sY, tid);
+            put_chunk16<false>(nx, t1, M, K, r0, kc * kAnyTile, sX, tid);
+            put_chunk16<true>(ny, t2, N, K, cb * kAnyTile, kc * kAnyTile, sY, tid);
             int cb2 = cb, kc2 = kc + 1;
             if (kc2 == nkc) { kc2 = 0; ++cb2; }
             if (step + 1 < steps) {                                    // in flight under the matrix instructions
@@ -178,10 +205,11 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
             __syncthreads();
 #pragma unroll
             for (int ks = 0; ks < kAnyTile / 32; ++ks) {
-                const u32x4 av = *reinterpret_cast<const u32x4 *>(xa + ks * 64);
+                const u32x4 av = t1 ? lds_tr8(xt + ks * 32 * kAnyPitch) : *reinterpret_cast<const u32x4 *>(xa + ks * 64);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const u32x4 bv = *reinterpret_cast<const u32x4 *>(ya + t * kAnyPitch + ks * 64);
+                    const u32x4 bv = t2 ? lds_tr8(yt + ks * 32 * kAnyPitch + 32 * t)
+                                        : *reinterpret_cast<const u32x4 *>(ya + t * kAnyPitch + ks * 64);
                     acc[t] = Elem<DT>::mfma(av, bv, acc[t]);
                 }
             }
