@@ -114,6 +114,20 @@ def test_long_segments_many_key_blocks(dev):
     run(dev, [70], [2000], [64], 1, torch.float16, 1.0, sigma=2.0, seed=3)
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
+def test_random_batches(dev, seed):
+    # random batches: segment counts, heights, widths and head dimensions drawn anew (multiples of 8 or anything),
+    # with empty segments among them; both strip counts and every head-dimension build come up over the seeds
+    rng = np.random.default_rng(seed)
+    nseg = int(rng.integers(1, 40))
+    tall = seed % 2 == 0
+    M = rng.integers(0, 700 if tall else 150, nseg); N = rng.integers(0, 400, nseg)
+    kmax = int(rng.choice([16, 32, 64, 96, 128]))
+    K = rng.integers(1, kmax // 8 + 1, nseg) * 8 if seed % 3 else rng.integers(1, kmax + 1, nseg)
+    dtype = torch.float16 if seed % 2 else torch.bfloat16
+    run(dev, M, N, K, int(rng.integers(1, 4)), dtype, float(rng.uniform(0.05, 0.3)), seed=seed)
+
+
 def test_launch_without_the_host_summary(dev):
     M = [33, 5, 300, 64]; N = [40, 200, 70, 64]; K = [64, 128, 32, 72]
     run(dev, M, N, K, 2, torch.float16, 0.125, summary=False)
