@@ -30,6 +30,8 @@
 // per store instruction.  The pieces at the two ends of a row that the windows cannot cover whole are
 // written by one unaligned 16-byte store each (columns [0, 8) and [N-8, N); overlapping pieces carry
 // identical values).
+#include <stdlib.h>
+
 #include <algorithm>
 #include <type_traits>
 
@@ -558,8 +560,17 @@ int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, c
                      hipStream_t stream) {
     if (!info || info->max_K > 128 || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
     if (slots <= 0) return BA_OK;
-    const int64_t z = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRbRows - 1) / kRbRows));
     const int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
+    // Workgroups per pair (workgroup z of a pair takes its row blocks z, z + Z, ..): enough for about three
+    // workgroups per compute unit over the launch, at most one per row block of the tallest segment.  One
+    // workgroup per row block was the rule before: between two workgroups a compute unit waits about 10 us for the
+    // stores of the one to drain and the next to be dispatched, and pairs with fewer row blocks than Z leave
+    // workgroups that start only to end (16 x 16 pairs of 4 .. 16 row blocks: 2704 + 1392 workgroups, 1.89 ms;
+    // with Z = 3 768 workgroups, 1.83 ms; the product alone 1.30 -> 1.20 ms).  BLOCKEDATTN_ROWBLOCK_Z overrides.
+    static const int forced_z = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK_Z"); return e ? atoi(e) : 0; }();
+    const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRbRows - 1) / kRbRows));
+    int64_t z = std::min<int64_t>(z_max, (3 * 256 + pairs - 1) / pairs);
+    if (forced_z > 0) z = std::min<int64_t>(z_max, forced_z);
     const int64_t groups = pairs * z;
     if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
     int st;
