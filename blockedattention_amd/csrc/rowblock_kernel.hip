@@ -84,12 +84,14 @@ __device__ __forceinline__ u32x4 ring_read16(const unsigned char *row, int pos) 
 }
 
 template <int DT, bool FUSED>
-__global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunArgs a, int zdim) {
+__global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunArgs a, int zdim, int weave) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const unsigned block = blockIdx.x;
     const int die = block % kDies, slot = block / kDies;
-    const int pair = (slot / zdim) * kDies + die;
-    const int z0 = slot % zdim;
+    // `weave` pairs of a die take turns in the die's slots (pair fastest, then the pair's workgroups)
+    const int turn = slot % (zdim * weave);
+    const int pair = ((slot / (zdim * weave)) * weave + turn % weave) * kDies + die;
+    const int z0 = turn / weave;
     const int H = (int)a.H;
     const PlanRO pv = plan_ro(a.plan, a.nseg);
     if (!header_ok(a)) {
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
     }
     // Workgroup -> (list entry, head, row block).  Consecutive workgroup ids go to the eight dies in turn, each with
     // its own L2; all row blocks of one (entry, head) pair read the same B_g, so they run on ONE die, one after
-    // the other: id = 8 slot + die works on pair 8 (slot / zdim) + die, row block slot % zdim.  The pairs are
+    // the other: id = 8 slot + die works on pair 8 (slot / zdim) + die, row block slot % zdim (weave = 1).  The pairs are
     // numbered entry-major with the entries in order of DECREASING work (M N): the long workgroups start first,
     // the short ones fill the gaps at the end, and every die gets two heads in eight of every entry.
     const int entries = a.list < 0 ? a.nseg : (int)((ConstHdr)(uintptr_t)a.plan)->totals[a.list];
@@ -546,11 +548,11 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
 }
 
 template <int DT, bool FUSED>
-static int launch_rb(const RunArgs &args, unsigned groups, int zdim, hipStream_t stream) {
+static int launch_rb(const RunArgs &args, unsigned groups, int zdim, int weave, hipStream_t stream) {
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&rowblock_kernel<DT, FUSED>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes);
     if (attr != hipSuccess) return BA_ERR_LAUNCH;
-    hipLaunchKernelGGL((rowblock_kernel<DT, FUSED>), dim3(groups), dim3(kRbThreads), kRbLdsBytes, stream, args, zdim);
+    hipLaunchKernelGGL((rowblock_kernel<DT, FUSED>), dim3(groups), dim3(kRbThreads), kRbLdsBytes, stream, args, zdim, weave);
     return BA_OK;
 }
 
@@ -560,24 +562,30 @@ int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, c
                      hipStream_t stream) {
     if (!info || info->max_K > 128 || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
     if (slots <= 0) return BA_OK;
-    const int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
-    // Workgroups per pair (workgroup z of a pair takes its row blocks z, z + Z, ..): enough for about three
-    // workgroups per compute unit over the launch, at most one per row block of the tallest segment.  One
-    // workgroup per row block was the rule before: between two workgroups a compute unit waits about 10 us for the
-    // stores of the one to drain and the next to be dispatched, and pairs with fewer row blocks than Z leave
-    // workgroups that start only to end (16 x 16 pairs of 4 .. 16 row blocks: 2704 + 1392 workgroups, 1.89 ms;
-    // with Z = 3 768 workgroups, 1.83 ms; the product alone 1.30 -> 1.20 ms).  BLOCKEDATTN_ROWBLOCK_Z overrides.
+    int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
+    // Workgroups per pair Z (workgroup z of a pair takes its row blocks z, z + Z, ..) and pairs of a die that take
+    // turns in the grid.  Sixteen workgroups of one pair that start together fetch the same lines of B_g at the same
+    // moment, and a compute unit waits about 10 us between two workgroups (stores of the one draining, dispatch of
+    // the next), also for the workgroups that pairs with fewer row blocks than Z leave empty.  Measured on 16 x 16
+    // pairs of 4 .. 16 row blocks, fused / product alone: Z = 16 1874 / 1307 us; two pairs taking turns 1795 / 1303;
+    // Z = 3 (about three workgroups per compute unit) 1813 / 1201, but then ten pairs are in flight per die, B_g
+    // leaves the die's L2 between a workgroup's passes and the launch reads 1.9 GB instead of 0.6.
+    // Hence: fused, one workgroup per row block and two pairs taking turns; the product alone, Z = 3 x 256 / pairs.
+    // BLOCKEDATTN_ROWBLOCK_Z and BLOCKEDATTN_ROWBLOCK_WEAVE override.
     static const int forced_z = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK_Z"); return e ? atoi(e) : 0; }();
+    static const int forced_w = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK_WEAVE"); return e ? atoi(e) : 0; }();
     const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRbRows - 1) / kRbRows));
-    int64_t z = std::min<int64_t>(z_max, (3 * 256 + pairs - 1) / pairs);
+    int64_t z = fused ? z_max : std::min<int64_t>(z_max, (3 * 256 + pairs - 1) / pairs);
     if (forced_z > 0) z = std::min<int64_t>(z_max, forced_z);
+    const int64_t weave = std::max<int64_t>(1, std::min<int64_t>(forced_w > 0 ? forced_w : (fused ? 2 : 1), pairs / kDies));
+    pairs = (pairs / kDies + weave - 1) / weave * weave * kDies;       // whole turns
     const int64_t groups = pairs * z;
     if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
     int st;
-    if (dtype == BA_F16) st = fused ? launch_rb<0, true>(args, (unsigned)groups, (int)z, stream)
-                                    : launch_rb<0, false>(args, (unsigned)groups, (int)z, stream);
-    else if (dtype == BA_BF16) st = fused ? launch_rb<1, true>(args, (unsigned)groups, (int)z, stream)
-                                          : launch_rb<1, false>(args, (unsigned)groups, (int)z, stream);
+    if (dtype == BA_F16) st = fused ? launch_rb<0, true>(args, (unsigned)groups, (int)z, (int)weave, stream)
+                                    : launch_rb<0, false>(args, (unsigned)groups, (int)z, (int)weave, stream);
+    else if (dtype == BA_BF16) st = fused ? launch_rb<1, true>(args, (unsigned)groups, (int)z, (int)weave, stream)
+                                          : launch_rb<1, false>(args, (unsigned)groups, (int)z, (int)weave, stream);
     else return BA_ERR_UNSUPPORTED;
     if (st != BA_OK) return st;
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
