@@ -56,6 +56,9 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
 // BA_ERR_UNSUPPORTED when the plan summary is missing or does not fit; the caller then takes launch_tiles.
 int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                      hipStream_t stream);
+// The pipelined row-block kernel (rowpipe_kernel.hip): the fused pair over the same list, two sweeps of adjacent
+// row blocks sharing one stream of B_g.  Same conditions as launch_rowblocks.
+int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_info *info, hipStream_t stream);
 // fp16 / bf16 in any layout and alignment (gemm_any16.hip: both operands staged through LDS, MFMA)
 int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 // fp32, fp64 and the integer types (gemm_generic.hip); dtype: ba_dtype

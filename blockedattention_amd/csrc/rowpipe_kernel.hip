@@ -1,0 +1,568 @@
+// The pipelined row-block kernel: softmax(scale * A_g B_g^T) for large segments (the tile kernel's class,
+// N > 256) with K <= 128 and 16-bit results, written so that the two sweeps of the softmax share one stream
+// of B_g through LDS.
+//
+// One workgroup = 8 wavefronts in two SETS of four.  A set works on one block of 256 rows (wavefront q of the
+// set: rows 64 q .. 64 q + 63, four MFMA row tiles, A fragments in registers) and goes through the columns
+// twice: sweep 1 sums exp2((s - R) c) per row, sweep 2 recomputes the scores and writes
+// exp2(s c - R c - log2(sum)).  The sets are one sweep apart: while set X runs sweep 2 of row block b, set Y
+// runs sweep 1 of row block b + 1 ON THE SAME CHUNKS of B_g (64 columns x 128 k, 16 KiB, four LDS stages).
+// What that buys, against one sweep after the other in every wavefront:
+//   * a wavefront of 64 rows reads each B fragment once for four matrix instructions; with 32 rows the LDS
+//     operand reads alone keep the LDS busy for as long as the matrix instructions take;
+//   * every chunk is fetched from L2 once for both sweeps;
+//   * the wavefronts that store (sweep 2) issue no loads, and the wavefronts that fill the stages (sweep 1, or
+//     idle) issue no stores: the in-order memory counter of a filling wavefront holds nothing but fills;
+//   * at any time half of the wavefronts of a compute unit store, so the result leaves at an even rate.
+//
+// A wavefront's 64 x 64 block of a chunk is computed as two halves of 32 columns (column tile ct of the chunk
+// takes the B rows 4 j + ct; half h = tiles 2h, 2h + 1), into two accumulator sets that alternate: the 32
+// matrix instructions of one half are threaded, one by one, through the softmax arithmetic of the half before
+// (per score: x = s c + ref, exp2 of the previous x, use of the exponential before that).  A lane (j = lane %
+// 16, rg = lane / 16) holds rows 16 rt + 4 rg + i and, per half, the two consecutive columns 4 j + 2 h + {0, 1}.
+//
+// Sweep 1 measures every score against R = the row's maximum over the FIRST half chunk (the sum then holds a
+// term 1 and cannot vanish).  Should a later score exceed R by more than the exponent range, the sum overflows;
+// that is seen when the sweep ends, and the set then repeats the block in two sweeps that cannot overflow (row
+// maximum over all columns, then the sum against it) while the other set waits for it where it must.
+//
+// Stores: as in the row-block kernel, a wavefront's results pass through a ring in LDS (one row of 128 columns
+// per result row) and leave as line-aligned 128-byte windows, eight lanes x 16 bytes per row, so that every
+// 128-byte line of the result is written whole and once; the row ends that no window covers whole are written
+// by one unaligned 16-byte store each.  The ring of wavefront q is used by whichever set is in sweep 2.
+#include <stdlib.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "tile_body.hpp"
+
+namespace ba {
+
+constexpr int kRpWaves = 8;
+constexpr int kRpThreads = 64 * kRpWaves;
+constexpr int kRpSetWaves = 4;
+constexpr int kRpRT = 4;                                  // MFMA row tiles per wavefront
+constexpr int kRpWaveRows = 16 * kRpRT;                   // 64
+constexpr int kRpBlockRows = kRpSetWaves * kRpWaveRows;   // 256 rows per set and step
+constexpr int kRpCols = 64;                               // columns per chunk
+constexpr int kRpStageBytes = kRpCols * 256;              // 16 KiB: 64 rows of B_g x 128 k
+constexpr int kRpStages = 4;
+constexpr int kRpFillInsts = kRpStageBytes / 1024 / kRpSetWaves;   // global->LDS instructions per filling wavefront and chunk (4)
+constexpr int kRpStoreInsts = kRpWaveRows / 8;            // window stores per wavefront and chunk (8)
+constexpr int kRpRingPitch = 288;                         // 128 columns + a copy of the first 16 behind them
+constexpr int kRpRingBytes = kRpWaveRows * kRpRingPitch;  // per wavefront of a set
+constexpr int kRpFlagOffset = kRpStages * kRpStageBytes + kRpSetWaves * kRpRingBytes;
+constexpr int kRpLdsBytes = kRpFlagOffset + 64;
+constexpr uint32_t kRpOutOfRange = 0x80000000u;           // byte offset no segment reaches (areas are below 2^31 bytes)
+
+enum RpRole : int { kRoleNone = 0, kRoleSum = 1, kRoleMax = 2, kRoleSumSafe = 3, kRoleOut = 4 };
+
+__device__ __forceinline__ void rp_wait_vm_upto(int n) {  // n in {0, 4, 8}, wave-uniform
+    if (n >= 8) wait_vm<8>();
+    else if (n >= 4) wait_vm<4>();
+    else wait_vm<0>();
+}
+
+// Sixteen bytes of a ring row starting at byte `pos` (any even value below 256): five aligned words, shifted.
+__device__ __forceinline__ u32x4 rp_ring_read16(const unsigned char *row, int pos) {
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(row + (pos & ~3));
+    const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
+    const uint32_t sh = (uint32_t)(pos & 2) * 8;
+    return u32x4{__builtin_amdgcn_alignbit(d1, d0, sh), __builtin_amdgcn_alignbit(d2, d1, sh),
+                 __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh)};
+}
+
+template <int DT>
+__global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int zdim, int weave) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    const unsigned block = blockIdx.x;
+    const int die = block % kDies, slot = block / kDies;
+    // `weave` pairs of a die take turns in the die's slots (pair fastest, then the pair's workgroups)
+    const int turn = slot % (zdim * weave);
+    const int pair = ((slot / (zdim * weave)) * weave + turn % weave) * kDies + die;
+    const int z0 = turn / weave;
+    const int H = (int)a.H;
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
+    if (!header_ok(a)) {
+        if (!(a.flags & kFlagQuiet) && block == 0 && threadIdx.x == 0)
+            atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+        return;
+    }
+    // Workgroup -> (list entry, head, share of the row blocks).  Consecutive workgroup ids go to the eight dies in
+    // turn, each with its own L2; all workgroups of one (entry, head) pair read the same B_g, so they run on ONE
+    // die.  The pairs are numbered entry-major with the entries in order of DECREASING work (M N).
+    const int entries = a.list < 0 ? a.nseg : (int)((ConstHdr)(uintptr_t)a.plan)->totals[a.list];
+    if (entries <= 0 || pair >= entries * H) return;
+    const int h = pair % H;
+    int entry = pair / H;
+    if (entries <= 64) {
+        const int lane0 = lane_id();
+        const ConstSeg list = pv.recs + (int64_t)(a.list + 1) * plan_cap(a.nseg);
+        int64_t work = -1;
+        if (lane0 < entries) {
+            const SegRec *r = reinterpret_cast<const SegRec *>((uintptr_t)(list + lane0));
+            work = (int64_t)r->M * r->N;
+        }
+        int rank = 0;
+        for (int e = 0; e < entries; ++e) {
+            const int64_t other = uniform64(__shfl(work, e));
+            rank += (other > work || (other == work && e < lane0)) ? 1 : 0;
+        }
+        const uint64_t hit = __ballot(lane0 < entries && rank == entry);
+        entry = hit ? (int)__builtin_ctzll(hit) : entries;
+        if (entry >= entries) return;
+    }
+    bool valid;
+    const Seg s = load_listed(pv, entry, h, a, valid);
+    if (!valid || !tile_segment(s.kind, s.N, s.K)) return;
+    const int M = s.M, N = s.N, K = s.K;
+    const int nrb = (M + kRpBlockRows - 1) / kRpBlockRows;
+    const int b_begin = (int)((int64_t)z0 * nrb / zdim), b_end = (int)((int64_t)(z0 + 1) * nrb / zdim);
+    if (b_begin >= b_end) return;
+    const int ncb = (N + kRpCols - 1) / kRpCols;
+    if (K > 128 || ncb < kRpStages) {            // the launch was sized for another plan
+        if (z0 == 0 && threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+        return;
+    }
+    const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
+    const int wave = uniform((int)(threadIdx.x >> 6));
+    const int set = wave >> 2, wq = wave & 3;
+    const SegRes res = make_res(s, a.A, a.B);
+    const char *bseg = reinterpret_cast<const char *>((const uint16_t *)a.B + s.b);
+    char *oseg = reinterpret_cast<char *>(a.out) + s.o * 2;
+    const __amdgpu_buffer_rsrc_t out_res =
+        __builtin_amdgcn_make_buffer_rsrc(oseg, 0, (int)((uint32_t)M * (uint32_t)N * 2u), kRsrcFlags);
+    const uint32_t out_phase = (uint32_t)(uintptr_t)oseg;   // low address bits decide the line phase of a row
+    unsigned char *ring = lds + kRpStages * kRpStageBytes + wq * kRpRingBytes;
+    volatile int *flags = reinterpret_cast<volatile int *>(lds + kRpFlagOffset);   // [parity of the step][set]
+
+    const int ksteps = (K + 31) >> 5;
+    const int kpieces = K >> 3;                            // 16-byte pieces per row of B_g
+    const float c_signed = a.scale * kLog2e;
+    const bool negate = c_signed < 0.f;                    // |scale| on negated scores
+    const float c = __builtin_fabsf(c_signed);
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+    // Stale or never written LDS must not reach a matrix instruction as NaN bits: pieces past K are never
+    // filled, so the stages start as zeros.
+    for (int off = (int)threadIdx.x * 16; off < kRpStages * kRpStageBytes; off += kRpThreads * 16)
+        *reinterpret_cast<u32x4 *>(lds + off) = zero4;
+    if (threadIdx.x < 4) flags[threadIdx.x] = 0;
+    __syncthreads();                                      // no fill may land under a late zero
+
+    // Fill of one chunk by the four wavefronts of a set: instruction i (0..15) covers LDS rows 4i .. 4i+3 of the
+    // stage; lane l writes row 4i + l/16, slot l%16, which holds piece (l%16) ^ (i%16) of that row.  Wavefront q
+    // issues i = q + 4 n.  Rows past N (ragged last chunk) fetch row N - 1 instead, so that every instruction is
+    // issued whatever the shape and the count of outstanding fills is known; lanes whose piece lies past K stay
+    // idle (every instruction has lanes with a piece, K >= 8).  Written as assembly on purpose: the compiler
+    // orders every LDS access behind ALL outstanding vector memory operations once it has seen a load into LDS.
+    // (instruction i = q + 4n: piece = (l%16 ^ q) ^ 4n, row 4q + l/16 + 16n)
+    const int fill_p0 = (lane & 15) ^ wq;
+    const uint32_t fill_row = (uint32_t)((4 * wq + (lane >> 4)) * K) * 2u;
+    auto fill = [&](int cbi, int stage) __attribute__((always_inline)) {
+        const int cb = cbi * kRpCols;
+        const char *base = reinterpret_cast<const char *>((uintptr_t)uniform64((int64_t)(uintptr_t)(bseg + (size_t)cb * K * 2)));
+        const bool whole = cb + kRpCols <= N;
+#pragma unroll
+        for (int n = 0; n < kRpFillInsts; ++n) {
+            const int i = wq + kRpSetWaves * n;
+            const uint32_t dst = (uint32_t)uniform((int)(uint32_t)(uintptr_t)(lds + stage * kRpStageBytes + i * 1024));
+            const int piece = fill_p0 ^ (4 * n);
+            uint32_t off = fill_row + (uint32_t)(32 * n * K + 16 * piece);
+            if (!whole) {
+                const int r = min(4 * i + (lane >> 4), N - 1 - cb);
+                off = (uint32_t)(r * K + piece * 8) * 2u;
+            }
+            if (piece < kpieces) {
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                             :: "v"(off), "s"(base), "s"(dst) : "memory", "m0");
+            }
+        }
+    };
+    // operand read offsets of this lane inside a stage: row 4j + ct, piece 4ks + rg at slot (4ks + rg) ^ j
+    // (k-step ks flips bits 2..3 of the slot: offset of k-step 0 exclusive-or 64 ks)
+    const int boff0 = 1024 * j + 16 * (rg ^ j);
+
+    // ---- per-wavefront state of the block the set works on
+    u32x4 af[kRpRT][4];                        // A fragments [rt][ks]: row 16 rt + j, k = 32 ks + 8 rg ..
+    float ref[kRpRT][4];                       // sweep 1: -R c; sweep 2: -R c - log2(sum)
+    float sum[kRpRT][4];                       // sweep 1: running sum; maximum sweep: running maximum
+    f32x4 acc[2][kRpRT][2];                    // [half][rt][column tile of the half]
+    uint32_t v0[kRpStoreInsts];                // sweep 2: byte offset of the lane's piece of window 0 inside the segment's result
+    uint32_t rn2 = 0;                          // ... and of the lane's first row (instruction 0)
+    int row0 = 0;
+    bool active = false;
+    const int q8 = lane & 7;
+    const unsigned char *rbase0 = ring + (lane >> 3) * kRpRingPitch;
+
+    auto load_block = [&](int blk) __attribute__((always_inline)) {
+        row0 = blk * kRpBlockRows + wq * kRpWaveRows;
+        active = row0 < M;
+#pragma unroll
+        for (int rt = 0; rt < kRpRT; ++rt) {
+            const int voff = ((row0 + 16 * rt + j) * K + rg * 8) * 2;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                u32x4 v = zero4;
+                if (ks < ksteps) {
+                    v = __builtin_amdgcn_raw_buffer_load_b128(res.a, voff + ks * 64, 0, 0);
+                    if (ks * 32 + rg * 8 >= K) v = zero4;            // ragged last k-step
+                    if (negate) v ^= u32x4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+                }
+                af[rt][ks] = v;
+            }
+        }
+    };
+    // store lanes: instruction t writes rows 8t + lane/8, piece lane%8 of the row's aligned window
+    auto store_lanes = [&]() __attribute__((always_inline)) {
+        rn2 = 2u * (uint32_t)((row0 + (lane >> 3)) * N);
+#pragma unroll
+        for (int t = 0; t < kRpStoreInsts; ++t) {
+            const int rho = row0 + 8 * t + (lane >> 3);
+            const bool row_ok = rho < M;
+            const int rn = row_ok ? rho * N : 0;
+            const int d = (int)(((out_phase + 2u * (uint32_t)rn) & 127u) >> 1);     // columns before the row's first line boundary
+            v0[t] = row_ok ? (uint32_t)(2 * (rn + 8 * q8 - d)) : kRpOutOfRange;
+        }
+    };
+    // ring byte of the lane's piece in window 0, 2 (8q - d) mod 256: what v0 holds beyond the start of the row
+    auto upos_of = [&](int t) __attribute__((always_inline)) {
+        return (int)((v0[t] - rn2 - (uint32_t)(16 * t * N)) & 255u);
+    };
+
+    // -------- out of the ring: one line-aligned 128-byte window per row and chunk
+    auto ring_copy_heads = [&](int first_row) __attribute__((always_inline)) {
+        // the first 32 bytes of sixteen ring rows once more behind the rows: pieces that start in a row's
+        // last 16 bytes continue there
+        const unsigned char *src = ring + (first_row + (lane >> 2)) * kRpRingPitch + (lane & 3) * 8;
+        *reinterpret_cast<u32x2 *>(const_cast<unsigned char *>(src) + 256) = *reinterpret_cast<const u32x2 *>(src);
+        asm volatile("" ::: "memory");
+    };
+    // interior chunk: the sixteen rows of row tile rt leave as soon as they are in the ring
+    auto ring_store_rows = [&](int cbi, auto rt_c) __attribute__((always_inline)) {
+        constexpr int rt = decltype(rt_c)::value;
+        if (cbi == 0 || cbi == ncb - 1) return;           // first and last chunk: ring_store_edge
+        asm volatile("" ::: "memory");                    // the reads below see the writes above (same wavefront, in order)
+        if ((cbi & 1) == 0) ring_copy_heads(16 * rt);
+        const int par = (cbi & 1) << 7;
+        const uint32_t adv = 128u * (uint32_t)cbi;        // the range check sees the vector offset only
+#pragma unroll
+        for (int t = 2 * rt; t < 2 * rt + 2; ++t) {
+            const u32x4 v = rp_ring_read16(rbase0 + t * 8 * kRpRingPitch, upos_of(t) ^ par);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, v0[t] == kRpOutOfRange ? kRpOutOfRange : v0[t] + adv, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+    };
+    // First or last chunk: pieces before column 0 or past column N are dropped, and the end pieces the windows
+    // cannot cover whole are written by one unaligned store each (lane l: row l).
+    auto ring_store_edge = [&](int cbi) __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");
+        if ((cbi & 1) == 0) { ring_copy_heads(0); ring_copy_heads(16); ring_copy_heads(32); ring_copy_heads(48); }
+        const int par = (cbi & 1) << 7;
+        const uint32_t adv = 128u * (uint32_t)cbi;
+        const int et_row = row0 + lane;
+        const uint32_t et_off = et_row < M ? (uint32_t)(2 * (et_row * N)) : kRpOutOfRange;
+        const unsigned char *et_base = ring + lane * kRpRingPitch;
+#pragma unroll
+        for (int t = 0; t < kRpStoreInsts; ++t) {
+            const int up = upos_of(t);
+            const u32x4 v = rp_ring_read16(rbase0 + t * 8 * kRpRingPitch, up ^ par);
+            const int col = (((up >> 1) + 64) & 127) - 64 + kRpCols * cbi;      // first column of the piece
+            const uint32_t voff = (col < 0 || col + 8 > N || v0[t] == kRpOutOfRange) ? kRpOutOfRange : v0[t] + adv;
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+        }
+        if (cbi == 0) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(et_base);          // columns [0, 8)
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, 0);
+        }
+        if (cbi == ncb - 1) {
+            // the window behind the last chunk (what is left of the rows), then columns [N-8, N)
+            const int par2 = (ncb & 1) << 7;
+#pragma unroll
+            for (int t = 0; t < kRpStoreInsts; ++t) {
+                const int up = upos_of(t);
+                const u32x4 v = rp_ring_read16(rbase0 + t * 8 * kRpRingPitch, up ^ par2);
+                const int col = (((up >> 1) + 64) & 127) - 64 + kRpCols * ncb;
+                const uint32_t voff = (col + 8 <= N && v0[t] != kRpOutOfRange) ? v0[t] + 128u * (uint32_t)ncb : kRpOutOfRange;
+                __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+            }
+            const u32x4 v = rp_ring_read16(et_base, (2 * (N - 8)) & 255);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off == kRpOutOfRange ? kRpOutOfRange : et_off + 2u * (uint32_t)(N - 8), 0, 0);
+        }
+        asm volatile("" ::: "memory");
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+
+    // -------- one half: the 32 matrix instructions of half HALF of the chunk in `stage` (when MFMA) into
+    // accumulator set HALF, with the arithmetic of the half before -- half 1 - HALF of chunk `cprev`, in the
+    // other accumulator set -- threaded between them, one score element per matrix instruction.
+    // MODE 0: matrix instructions only; kRoleSum: sum += w exp2(s c + ref); kRoleMax: running maximum;
+    // kRoleOut: exp2(s c + ref) into the ring (and, with HALF = 0, which completes chunk cprev, out of it).
+    auto half_body = [&](auto mode_c, auto half_c, auto mfma_c, int stage, int cprev) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode_c)::value;
+        constexpr int hb = decltype(half_c)::value, pb = 1 - hb;
+        constexpr bool MFMA = decltype(mfma_c)::value;
+        const unsigned char *sb = lds + stage * kRpStageBytes + 512 * hb;
+        const int colp = cprev * kRpCols + 4 * j + 2 * pb;     // first of the lane's two columns of the half before
+        float w[2];                                            // 0 for columns that do not exist (ragged last chunk)
+        w[0] = colp < N ? 1.f : 0.f;
+        w[1] = colp + 1 < N ? 1.f : 0.f;
+        unsigned char *wrow = ring + (4 * rg) * kRpRingPitch + ((cprev & 1) << 7) + (4 * j + 2 * pb) * 2;
+        u32x4 bf[2][2];
+        if constexpr (MFMA) {
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct) bf[0][ct] = *reinterpret_cast<const u32x4 *>(sb + boff0 + 256 * ct);
+        }
+        float xprev = 0.f, pprev = 0.f, plo = 0.f;
+        auto use = [&](auto e_c, float pval) {
+            constexpr int pe = decltype(e_c)::value, prt = pe >> 3, pi = (pe >> 1) & 3, pct = pe & 1;
+            if constexpr (MODE == kRoleSum) sum[prt][pi] = fmaf(pval, w[pct], sum[prt][pi]);
+            else if constexpr (MODE == kRoleMax) sum[prt][pi] = __builtin_fmaxf(sum[prt][pi], w[pct] != 0.f ? pval : -3.0e38f);
+            else if constexpr (MODE == kRoleOut) {
+                if constexpr (pct == 0) plo = pval;
+                else {
+                    *reinterpret_cast<uint32_t *>(wrow + (16 * prt + pi) * kRpRingPitch) = Elem<DT>::pack2(plo, pval);
+                    if constexpr (hb == 0 && (pe & 7) == 7)
+                        ring_store_rows(cprev, std::integral_constant<int, prt>{});   // the row tile is in the ring, both halves
+                }
+            }
+        };
+        auto power = [&](float x) { return MODE == kRoleMax ? x : __builtin_amdgcn_exp2f(x); };
+        auto element = [&](auto e_c) {
+            constexpr int e = decltype(e_c)::value, rt2 = e >> 3, i2 = (e >> 1) & 3, ct2 = e & 1;
+            if constexpr (e >= 2) use(std::integral_constant<int, e - 2>{}, pprev);
+            if constexpr (e >= 1) pprev = power(xprev);
+            const float sc = acc[pb][rt2][ct2][i2];
+            xprev = MODE == kRoleMax ? sc : fmaf(sc, c, ref[rt2][i2]);
+        };
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            if constexpr (MFMA) {
+                if (ks + 1 < 4) {
+#pragma unroll
+                    for (int ct = 0; ct < 2; ++ct)
+                        bf[(ks + 1) & 1][ct] = *reinterpret_cast<const u32x4 *>(sb + (boff0 ^ (64 * (ks + 1))) + 256 * ct);
+                }
+            }
+            auto group = [&](auto qd_c) {
+                constexpr int qd = decltype(qd_c)::value, rt = qd >> 1, ct = qd & 1;
+                if constexpr (MFMA)
+                    acc[hb][rt][ct] = Elem<DT>::mfma(af[rt][ks], bf[ks & 1][ct],
+                                                     ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[hb][rt][ct]);
+                if constexpr (MODE != 0) {
+                    if (ks == 0) element(std::integral_constant<int, 0 * 8 + qd>{});
+                    if (ks == 1) element(std::integral_constant<int, 1 * 8 + qd>{});
+                    if (ks == 2) element(std::integral_constant<int, 2 * 8 + qd>{});
+                    if (ks == 3) element(std::integral_constant<int, 3 * 8 + qd>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            group(I0{}); group(I1{}); group(I2{}); group(I3{});
+            group(std::integral_constant<int, 4>{}); group(std::integral_constant<int, 5>{});
+            group(std::integral_constant<int, 6>{}); group(std::integral_constant<int, 7>{});
+        }
+        if constexpr (MODE != 0) {
+            use(std::integral_constant<int, 30>{}, pprev);
+            pprev = power(xprev);
+            use(std::integral_constant<int, 31>{}, pprev);
+        }
+    };
+
+    // sweep 1, first half chunk: the reference of every row = its maximum over these 32 columns
+    auto stats_reference = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int rt = 0; rt < kRpRT; ++rt) {
+            float mx[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mx[i] = __builtin_fmaxf(acc[0][rt][0][i], acc[0][rt][1][i]);
+            row16_max4(mx);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ref[rt][i] = -__builtin_fmaxf(mx[i], -3.0e38f) * c;
+        }
+    };
+    // after the last chunk of sweep 1: row sums over the sixteen lanes; returns whether any is not finite
+    auto finish_stats = [&]() __attribute__((always_inline)) {
+        bool bad = false;
+#pragma unroll
+        for (int rt = 0; rt < kRpRT; ++rt) {
+            float sm[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sm[i] = sum[rt][i];
+            row16_sum4(sm);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                bad |= !(sm[i] <= 3.0e38f);
+                ref[rt][i] -= __builtin_amdgcn_logf(sm[i]);      // 1/sum goes into the exponent
+            }
+        }
+        return bad;
+    };
+    // after the maximum sweep: the reference of every row = its maximum over all columns
+    auto finish_max = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int rt = 0; rt < kRpRT; ++rt) {
+            float mx[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mx[i] = sum[rt][i];
+            row16_max4(mx);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ref[rt][i] = -__builtin_fmaxf(mx[i], -3.0e38f) * c;
+        }
+    };
+
+    // -------- the steps.  All of this is the same in every wavefront of the workgroup (scalar registers).
+    int role[2] = {kRoleNone, kRoleNone};
+    int next_block = b_begin;
+    int gpos = 0;                                          // chunks gone by since the workgroup started: stage = gpos % 4
+    bool first_step = true;
+    for (int step = 0;; ++step) {
+        // a set without work takes the next row block, unless the other set would then reach sweep 2 together with it
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            if (role[g] == kRoleNone && next_block < b_end && role[1 - g] != kRoleSum && role[1 - g] != kRoleSumSafe) {
+                role[g] = kRoleSum;
+                if (g == set) load_block(next_block);
+                ++next_block;
+            }
+        }
+        if (role[0] == kRoleNone && role[1] == kRoleNone) break;
+        const bool final_step = next_block >= b_end && (role[0] == kRoleNone || role[0] == kRoleOut) &&
+                                (role[1] == kRoleNone || role[1] == kRoleOut);
+        // the set that stores does not fill; of two sets that do not store, the idle one fills
+        const int filler_set = role[0] == kRoleOut ? 1 : role[1] == kRoleOut ? 0 : role[1] == kRoleNone ? 1 : 0;
+        const bool filler = set == filler_set;
+        const int my_role = role[set];
+        if (first_step) {
+            if (filler) {
+                for (int k = 0; k < kRpStages - 1; ++k) fill(k, k);
+                wait_vm<0>();
+            } else {
+                wait_vm<0>();                              // the A fragments
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            first_step = false;
+        }
+        // SYNC of iteration i: the filling wavefronts wait for their part of chunk i (requested three iterations
+        // ago, right behind that iteration's barrier; the fills of the two iterations since may stay in flight;
+        // the first three chunks of a step were complete before the step began), barrier (now everyone's part is
+        // there and nobody reads the stage of chunk i - 1 any more), request chunk i + 3 -- which, in any step but
+        // the workgroup's last, is a chunk of the next step once the end of B_g is near.
+        auto sync = [&](int i) __attribute__((always_inline)) {
+            if (filler && i >= kRpStages - 1) {
+                int later = 2 * kRpFillInsts;
+                if (final_step) later = kRpFillInsts * ((i + 1 < ncb ? 1 : 0) + (i + 2 < ncb ? 1 : 0));
+                rp_wait_vm_upto(later);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (filler && (!final_step || i + kRpStages - 1 < ncb)) {
+                int cbi = i + kRpStages - 1;
+                if (cbi >= ncb) cbi -= ncb;
+                fill(cbi, (gpos + i + kRpStages - 1) & (kRpStages - 1));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto run = [&](auto mode_c) __attribute__((always_inline)) {
+            constexpr int MODE = decltype(mode_c)::value;
+            using False = std::false_type;
+            using True = std::true_type;
+            // (a wavefront without rows only keeps the barriers and its fills: decided once, so that the accumulators
+            // are plainly defined before they are used in the branch that computes)
+            if (!active) {
+                for (int i = 0; i < ncb; ++i) sync(i);
+                return;
+            }
+            sync(0);
+            half_body(I0{}, I0{}, True{}, gpos & (kRpStages - 1), 0);
+            if (MODE == kRoleSum && my_role == kRoleSum) stats_reference();
+            half_body(mode_c, I1{}, True{}, gpos & (kRpStages - 1), 0);
+            for (int i = 1; i < ncb; ++i) {
+                sync(i);
+                const int stage = (gpos + i) & (kRpStages - 1);
+                half_body(mode_c, I0{}, True{}, stage, i - 1);
+                if (MODE == kRoleOut && i == 1) ring_store_edge(0);
+                half_body(mode_c, I1{}, True{}, stage, i);
+            }
+            half_body(mode_c, I0{}, False{}, 0, ncb - 1);
+            if (MODE == kRoleOut) ring_store_edge(ncb - 1);
+        };
+        // Every role keeps its state inside its own branch: what a sweep sets up, it alone uses (the sums of sweep 1,
+        // the store lanes of sweep 2), so none of it occupies registers in the other sweeps.
+        volatile int *fl = flags + 2 * (step & 1);
+        if (my_role == kRoleOut) {
+            store_lanes();
+            run(std::integral_constant<int, kRoleOut>{});
+        } else if (my_role == kRoleMax) {
+#pragma unroll
+            for (int rt = 0; rt < kRpRT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sum[rt][i] = -3.0e38f;
+            run(std::integral_constant<int, kRoleMax>{});
+            if (active) finish_max();
+        } else if (my_role == kRoleNone) {
+            for (int i = 0; i < ncb; ++i) sync(i);
+        } else {
+#pragma unroll
+            for (int rt = 0; rt < kRpRT; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sum[rt][i] = 0.f;
+            run(std::integral_constant<int, kRoleSum>{});
+            // the overflow verdict of sweep 1 goes to the whole workgroup through LDS
+            const bool bad = active && finish_stats();
+            if (my_role == kRoleSum && __ballot(bad) != 0 && lane == 0) fl[set] = 1;
+        }
+        gpos += ncb;
+        if (filler) wait_vm<0>();                         // the next step's first chunks are there before anyone takes over
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        const int over0 = uniform(fl[0]), over1 = uniform(fl[1]);
+        if (threadIdx.x == 0) { flags[2 * (1 - (step & 1))] = 0; flags[2 * (1 - (step & 1)) + 1] = 0; }
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const int over = g == 0 ? over0 : over1;
+            if (role[g] == kRoleSum) role[g] = over ? kRoleMax : kRoleOut;
+            else if (role[g] == kRoleMax) role[g] = kRoleSumSafe;
+            else if (role[g] == kRoleSumSafe) role[g] = kRoleOut;
+            else if (role[g] == kRoleOut) role[g] = kRoleNone;
+        }
+    }
+    wait_vm<0>();
+}
+
+template <int DT>
+static int launch_rp(const RunArgs &args, unsigned groups, int zdim, int weave, hipStream_t stream) {
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&rowpipe_kernel<DT>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kRpLdsBytes);
+    if (attr != hipSuccess) return BA_ERR_LAUNCH;
+    hipLaunchKernelGGL((rowpipe_kernel<DT>), dim3(groups), dim3(kRpThreads), kRpLdsBytes, stream, args, zdim, weave);
+    return BA_OK;
+}
+
+// Launches the pipelined row-block kernel over (list entry, head, share of the row blocks): the fused pair for
+// large segments with K <= 128 and 16-bit results.  Needs the plan summary.
+int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_info *info, hipStream_t stream) {
+    if (!info || info->max_K > 128 || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
+    if (slots <= 0) return BA_OK;
+    int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
+    static const int forced_z = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE_Z"); return e ? atoi(e) : 0; }();
+    static const int forced_w = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE_WEAVE"); return e ? atoi(e) : 0; }();
+    const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRpBlockRows - 1) / kRpBlockRows));
+    const int cus = device_cu_count();
+    int64_t z = std::min<int64_t>(z_max, std::max<int64_t>(1, (3 * (int64_t)cus + pairs - 1) / pairs));
+    if (forced_z > 0) z = std::min<int64_t>(z_max, forced_z);
+    const int64_t weave = std::max<int64_t>(1, std::min<int64_t>(forced_w > 0 ? forced_w : 1, pairs / kDies));
+    pairs = (pairs / kDies + weave - 1) / weave * weave * kDies;       // whole turns
+    const int64_t groups = pairs * z;
+    if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
+    int st;
+    if (dtype == BA_F16) st = launch_rp<0>(args, (unsigned)groups, (int)z, (int)weave, stream);
+    else if (dtype == BA_BF16) st = launch_rp<1>(args, (unsigned)groups, (int)z, (int)weave, stream);
+    else return BA_ERR_UNSUPPORTED;
+    if (st != BA_OK) return st;
+    return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+}
+
+}  // namespace ba
