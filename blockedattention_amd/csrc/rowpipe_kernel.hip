@@ -50,7 +50,8 @@ constexpr int kRpStageBytes = kRpCols * 256;              // 16 KiB: 64 rows of 
 constexpr int kRpStages = 4;
 constexpr int kRpFillInsts = kRpStageBytes / 1024 / kRpSetWaves;   // global->LDS instructions per filling wavefront and chunk (4)
 constexpr int kRpStoreInsts = kRpWaveRows / 8;            // window stores per wavefront and chunk (8)
-constexpr int kRpRingPitch = 288;                         // 128 columns + a copy of the first 16 behind them
+constexpr int kRpRingPitch = 296;                         // 128 columns + a copy of the first 16 behind them; 74 words: the
+                                                          // sixteen rows one 8-byte write instruction touches fall into sixteen bank pairs
 constexpr int kRpRingBytes = kRpWaveRows * kRpRingPitch;  // per wavefront of a set
 constexpr int kRpFlagOffset = kRpStages * kRpStageBytes + kRpSetWaves * kRpRingBytes;
 constexpr int kRpLdsBytes = kRpFlagOffset + 64;
@@ -64,14 +65,25 @@ __device__ __forceinline__ void rp_wait_vm_upto(int n) {  // n in {0, 4, 8}, wav
     else wait_vm<0>();
 }
 
-// Sixteen bytes of a ring row starting at byte `pos` (any even value below 256): five aligned words, shifted.
+// Sixteen bytes of a ring row starting at byte `pos` (any even value below 256): one LDS read at a 2-byte
+// alignment (the LDS takes wide accesses at any alignment; eight lanes reading eight consecutive pieces of a
+// row touch every bank once).
 __device__ __forceinline__ u32x4 rp_ring_read16(const unsigned char *row, int pos) {
-    const uint32_t *w = reinterpret_cast<const uint32_t *>(row + (pos & ~3));
-    const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
-    const uint32_t sh = (uint32_t)(pos & 2) * 8;
-    return u32x4{__builtin_amdgcn_alignbit(d1, d0, sh), __builtin_amdgcn_alignbit(d2, d1, sh),
-                 __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh)};
+    return *reinterpret_cast<const u32x4_unaligned *>(row + pos);
 }
+
+// A copy of a per-lane constant that the compiler cannot see through: what is derived from it inside a loop is
+// computed there (one or two instructions) instead of being kept in registers of its own across the loop.
+template <typename T> __device__ __forceinline__ T rp_fresh(T v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+#ifdef RP_X_NOSTORE
+#define RP_STORE(v, res, off) do { u32x4 v_ = (v); uint32_t o_ = (off); asm volatile("" :: "v"(v_), "v"(o_)); } while (0)
+#else
+#define RP_STORE(v, res, off) __builtin_amdgcn_raw_buffer_store_b128(v, res, off, 0, 0)
+#endif
 
 template <int DT>
 __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int zdim, int weave) {
@@ -141,7 +153,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     const int kpieces = K >> 3;                            // 16-byte pieces per row of B_g
     const float c_signed = a.scale * kLog2e;
     const bool negate = c_signed < 0.f;                    // |scale| on negated scores
-    const float c = __builtin_fabsf(c_signed);
+    const float c = __builtin_bit_cast(float, uniform(__builtin_bit_cast(int, __builtin_fabsf(c_signed))));   // in a scalar register
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
 
     // Stale or never written LDS must not reach a matrix instruction as NaN bits: pieces past K are never
@@ -152,49 +164,58 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     __syncthreads();                                      // no fill may land under a late zero
 
     // Fill of one chunk by the four wavefronts of a set: instruction i (0..15) covers LDS rows 4i .. 4i+3 of the
-    // stage; lane l writes row 4i + l/16, slot l%16, which holds piece (l%16) ^ (i%16) of that row.  Wavefront q
-    // issues i = q + 4 n.  Rows past N (ragged last chunk) fetch row N - 1 instead, so that every instruction is
-    // issued whatever the shape and the count of outstanding fills is known; lanes whose piece lies past K stay
-    // idle (every instruction has lanes with a piece, K >= 8).  Written as assembly on purpose: the compiler
-    // orders every LDS access behind ALL outstanding vector memory operations once it has seen a load into LDS.
-    // (instruction i = q + 4n: piece = (l%16 ^ q) ^ 4n, row 4q + l/16 + 16n)
-    const int fill_p0 = (lane & 15) ^ wq;
-    const uint32_t fill_row = (uint32_t)((4 * wq + (lane >> 4)) * K) * 2u;
-    auto fill = [&](int cbi, int stage) __attribute__((always_inline)) {
+    // stage; lane l writes row r = 4i + l/16, slot l%16, which holds piece (l%16) ^ (r%16) of that row (the sixteen
+    // lanes of an operand read take sixteen consecutive rows, 256 bytes apart: sixteen slots).  Wavefront q
+    // issues i = q + 4 n: row 4q + l/16 + 16 n, piece (l%16) ^ (4q + l/16) whatever n.  Rows past N (ragged last
+    // chunk) fetch row N - 1 instead, so that every instruction is issued whatever the shape and the count of
+    // outstanding fills is known.  Lanes whose piece lies past K stay idle: the instruction runs under a lane mask
+    // set INSIDE the assembly (a branch around it would split the body it is threaded into, and the compiler moves
+    // the arithmetic out of a split body).  Written as assembly on purpose: the compiler orders every LDS access
+    // behind ALL outstanding vector memory operations once it has seen a load into LDS.
+    const int fill_piece = (lane & 15) ^ (4 * wq + (lane >> 4));
+    const uint32_t fill_row = (uint32_t)((4 * wq + (lane >> 4)) * K + fill_piece * 8) * 2u;
+    uint64_t fill_mask = __ballot(fill_piece < kpieces);      // K = 0: no lane, and then no fill is issued at all
+    const bool fills_on = kpieces > 0;
+    auto fill_one = [&](auto n_c, int cbi, int stage) __attribute__((always_inline)) {
+        constexpr int n = decltype(n_c)::value;
         const int cb = cbi * kRpCols;
         const char *base = reinterpret_cast<const char *>((uintptr_t)uniform64((int64_t)(uintptr_t)(bseg + (size_t)cb * K * 2)));
-        const bool whole = cb + kRpCols <= N;
-#pragma unroll
-        for (int n = 0; n < kRpFillInsts; ++n) {
-            const int i = wq + kRpSetWaves * n;
-            const uint32_t dst = (uint32_t)uniform((int)(uint32_t)(uintptr_t)(lds + stage * kRpStageBytes + i * 1024));
-            const int piece = fill_p0 ^ (4 * n);
-            uint32_t off = fill_row + (uint32_t)(32 * n * K + 16 * piece);
-            if (!whole) {
-                const int r = min(4 * i + (lane >> 4), N - 1 - cb);
-                off = (uint32_t)(r * K + piece * 8) * 2u;
-            }
-            if (piece < kpieces) {
-                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                             :: "v"(off), "s"(base), "s"(dst) : "memory", "m0");
-            }
-        }
+        const int i = wq + kRpSetWaves * n;
+        const uint32_t dst = (uint32_t)uniform((int)(uint32_t)(uintptr_t)(lds + stage * kRpStageBytes + i * 1024));
+        // (the row clamp changes nothing in a whole chunk: two instructions, no branch)
+        const int r = min(4 * i + (lane >> 4), N - 1 - cb);
+        const uint32_t off = rp_fresh(fill_row) + (uint32_t)((r - 4 * wq - (lane >> 4)) * K) * 2u;
+#ifndef RP_X_NOFILL
+        uint64_t saved;
+        const uint64_t mask = fill_mask;
+        asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                     : "=&s"(saved) : "v"(off), "s"(base), "s"(dst), "s"(mask) : "memory", "m0");
+#endif
     };
-    // operand read offsets of this lane inside a stage: row 4j + ct, piece 4ks + rg at slot (4ks + rg) ^ j
-    // (k-step ks flips bits 2..3 of the slot: offset of k-step 0 exclusive-or 64 ks)
-    const int boff0 = 1024 * j + 16 * (rg ^ j);
+    auto fill = [&](int cbi, int stage) __attribute__((always_inline)) {
+        if (!fills_on) return;
+        fill_one(std::integral_constant<int, 0>{}, cbi, stage); fill_one(std::integral_constant<int, 1>{}, cbi, stage);
+        fill_one(std::integral_constant<int, 2>{}, cbi, stage); fill_one(std::integral_constant<int, 3>{}, cbi, stage);
+    };
+    // operand read offset of this lane inside a stage: column tile ct, row 16 ct + j, piece 4ks + rg at slot
+    // (4ks + rg) ^ j (k-step ks flips bits 2..3 of the slot: offset of k-step 0 exclusive-or 64 ks)
+    const int boff0 = 256 * j + 16 * (rg ^ j);
 
     // ---- per-wavefront state of the block the set works on
     u32x4 af[kRpRT][4];                        // A fragments [rt][ks]: row 16 rt + j, k = 32 ks + 8 rg ..
-    float ref[kRpRT][4];                       // sweep 1: -R c; sweep 2: -R c - log2(sum)
-    float sum[kRpRT][4];                       // sweep 1: running sum; maximum sweep: running maximum
-    f32x4 acc[2][kRpRT][2];                    // [half][rt][column tile of the half]
+    float ref[kRpRT];                          // of row 16 rt + j; sweep 1: -R c; sweep 2: -R c - log2(sum)
+    float sum[kRpRT];                          // sweep 1: running sum over the lane's columns; maximum sweep: running maximum
+    f32x4 acc[2][kRpRT];                       // [quarter % 2][rt]: columns 4 rg + i of the quarter's column tile
     uint32_t v0[kRpStoreInsts];                // sweep 2: byte offset of the lane's piece of window 0 inside the segment's result
-    uint32_t rn2 = 0;                          // ... and of the lane's first row (instruction 0)
+    int upos[kRpStoreInsts];                   // ... and ring byte of that piece: 2 (8q - d) mod 256
     int row0 = 0;
     bool active = false;
     const int q8 = lane & 7;
-    const unsigned char *rbase0 = ring + (lane >> 3) * kRpRingPitch;
+    // (byte offsets inside the workgroup's LDS)
+    const int ring_o = kRpStages * kRpStageBytes + wq * kRpRingBytes;
+    const int rbase_o = ring_o + (lane >> 3) * kRpRingPitch;                    // store lanes: row lane / 8 of a group of eight
+    const int ringw_o = ring_o + j * kRpRingPitch + 8 * rg;                     // ring writes: row j, columns 4 rg ..
 
     auto load_block = [&](int blk) __attribute__((always_inline)) {
         row0 = blk * kRpBlockRows + wq * kRpWaveRows;
@@ -214,51 +235,38 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             }
         }
     };
-    // store lanes: instruction t writes rows 8t + lane/8, piece lane%8 of the row's aligned window
+    // store lanes: instruction t writes rows 8t + lane/8, piece lane%8 of the row's aligned window.  A row without
+    // a store keeps its offset out of range: the marker plus any advance stays above 2^31.
     auto store_lanes = [&]() __attribute__((always_inline)) {
-        rn2 = 2u * (uint32_t)((row0 + (lane >> 3)) * N);
 #pragma unroll
         for (int t = 0; t < kRpStoreInsts; ++t) {
             const int rho = row0 + 8 * t + (lane >> 3);
             const bool row_ok = rho < M;
             const int rn = row_ok ? rho * N : 0;
             const int d = (int)(((out_phase + 2u * (uint32_t)rn) & 127u) >> 1);     // columns before the row's first line boundary
+            upos[t] = (16 * q8 - 2 * d) & 255;
             v0[t] = row_ok ? (uint32_t)(2 * (rn + 8 * q8 - d)) : kRpOutOfRange;
         }
     };
-    // ring byte of the lane's piece in window 0, 2 (8q - d) mod 256: what v0 holds beyond the start of the row
-    auto upos_of = [&](int t) __attribute__((always_inline)) {
-        return (int)((v0[t] - rn2 - (uint32_t)(16 * t * N)) & 255u);
-    };
 
-    // -------- out of the ring: one line-aligned 128-byte window per row and chunk
-    auto ring_copy_heads = [&](int first_row) __attribute__((always_inline)) {
-        // the first 32 bytes of sixteen ring rows once more behind the rows: pieces that start in a row's
-        // last 16 bytes continue there
-        const unsigned char *src = ring + (first_row + (lane >> 2)) * kRpRingPitch + (lane & 3) * 8;
-        *reinterpret_cast<u32x2 *>(const_cast<unsigned char *>(src) + 256) = *reinterpret_cast<const u32x2 *>(src);
-        asm volatile("" ::: "memory");
+    // -------- out of the ring: one line-aligned 128-byte window per row and chunk.  Interior chunk: the sixteen
+    // rows of row tile rt leave once they are in the ring, as two store instructions of eight rows; the LDS read of
+    // one is issued a few matrix instructions before its store (load / store+load / store, spread by the caller).
+    u32x4 ring_ld = {0u, 0u, 0u, 0u};
+    auto ring_load = [&](int cbi, auto t_c) __attribute__((always_inline)) {
+        constexpr int t = decltype(t_c)::value;
+        asm volatile("" ::: "memory");                    // the read sees the writes above (same wavefront, in order)
+        ring_ld = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ ((cbi & 1) << 7));
     };
-    // interior chunk: the sixteen rows of row tile rt leave as soon as they are in the ring
-    auto ring_store_rows = [&](int cbi, auto rt_c) __attribute__((always_inline)) {
-        constexpr int rt = decltype(rt_c)::value;
-        if (cbi == 0 || cbi == ncb - 1) return;           // first and last chunk: ring_store_edge
-        asm volatile("" ::: "memory");                    // the reads below see the writes above (same wavefront, in order)
-        if ((cbi & 1) == 0) ring_copy_heads(16 * rt);
-        const int par = (cbi & 1) << 7;
-        const uint32_t adv = 128u * (uint32_t)cbi;        // the range check sees the vector offset only
-#pragma unroll
-        for (int t = 2 * rt; t < 2 * rt + 2; ++t) {
-            const u32x4 v = rp_ring_read16(rbase0 + t * 8 * kRpRingPitch, upos_of(t) ^ par);
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, v0[t] == kRpOutOfRange ? kRpOutOfRange : v0[t] + adv, 0, 0);
-        }
+    auto ring_store = [&](int cbi, auto t_c) __attribute__((always_inline)) {
+        constexpr int t = decltype(t_c)::value;
+        RP_STORE(ring_ld, out_res, v0[t] + 128u * (uint32_t)cbi);        // (the range check sees the vector offset only)
         asm volatile("" ::: "memory");
     };
     // First or last chunk: pieces before column 0 or past column N are dropped, and the end pieces the windows
     // cannot cover whole are written by one unaligned store each (lane l: row l).
     auto ring_store_edge = [&](int cbi) __attribute__((always_inline)) {
         asm volatile("" ::: "memory");
-        if ((cbi & 1) == 0) { ring_copy_heads(0); ring_copy_heads(16); ring_copy_heads(32); ring_copy_heads(48); }
         const int par = (cbi & 1) << 7;
         const uint32_t adv = 128u * (uint32_t)cbi;
         const int et_row = row0 + lane;
@@ -266,29 +274,27 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         const unsigned char *et_base = ring + lane * kRpRingPitch;
 #pragma unroll
         for (int t = 0; t < kRpStoreInsts; ++t) {
-            const int up = upos_of(t);
-            const u32x4 v = rp_ring_read16(rbase0 + t * 8 * kRpRingPitch, up ^ par);
-            const int col = (((up >> 1) + 64) & 127) - 64 + kRpCols * cbi;      // first column of the piece
-            const uint32_t voff = (col < 0 || col + 8 > N || v0[t] == kRpOutOfRange) ? kRpOutOfRange : v0[t] + adv;
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+            const u32x4 v = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ par);
+            const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRpCols * cbi;      // first column of the piece
+            const uint32_t voff = (col < 0 || col + 8 > N) ? kRpOutOfRange : v0[t] + adv;
+            RP_STORE(v, out_res, voff);
         }
         if (cbi == 0) {
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(et_base);          // columns [0, 8)
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, 0);
+            const u32x4 v = rp_ring_read16(et_base, 0);                         // columns [0, 8)
+            RP_STORE(v, out_res, et_off);
         }
         if (cbi == ncb - 1) {
             // the window behind the last chunk (what is left of the rows), then columns [N-8, N)
             const int par2 = (ncb & 1) << 7;
 #pragma unroll
             for (int t = 0; t < kRpStoreInsts; ++t) {
-                const int up = upos_of(t);
-                const u32x4 v = rp_ring_read16(rbase0 + t * 8 * kRpRingPitch, up ^ par2);
-                const int col = (((up >> 1) + 64) & 127) - 64 + kRpCols * ncb;
-                const uint32_t voff = (col + 8 <= N && v0[t] != kRpOutOfRange) ? v0[t] + 128u * (uint32_t)ncb : kRpOutOfRange;
-                __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+                const u32x4 v = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ par2);
+                const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRpCols * ncb;
+                const uint32_t voff = col + 8 <= N ? v0[t] + 128u * (uint32_t)ncb : kRpOutOfRange;
+                RP_STORE(v, out_res, voff);
             }
             const u32x4 v = rp_ring_read16(et_base, (2 * (N - 8)) & 255);
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off == kRpOutOfRange ? kRpOutOfRange : et_off + 2u * (uint32_t)(N - 8), 0, 0);
+            RP_STORE(v, out_res, et_off + 2u * (uint32_t)(N - 8));
         }
         asm volatile("" ::: "memory");
     };
@@ -297,122 +303,140 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
+    using False = std::false_type;
+    using True = std::true_type;
 
-    // -------- one half: the 32 matrix instructions of half HALF of the chunk in `stage` (when MFMA) into
-    // accumulator set HALF, with the arithmetic of the half before -- half 1 - HALF of chunk `cprev`, in the
-    // other accumulator set -- threaded between them, one score element per matrix instruction.
-    // MODE 0: matrix instructions only; kRoleSum: sum += w exp2(s c + ref); kRoleMax: running maximum;
-    // kRoleOut: exp2(s c + ref) into the ring (and, with HALF = 0, which completes chunk cprev, out of it).
-    auto half_body = [&](auto mode_c, auto half_c, auto mfma_c, int stage, int cprev) __attribute__((always_inline)) {
+    // -------- one quarter: the 16 matrix instructions of column tile Q of the chunk in `stage` (when MFMA) into
+    // accumulator set Q % 2, with the arithmetic of the quarter before -- quarter (Q + 3) % 4 of chunk `cprev`, in
+    // the other accumulator set -- threaded between them, one score element per matrix instruction.
+    // MODE 0: matrix instructions only; kRoleSum: sum += exp2(s c + ref); kRoleMax: running maximum; kRoleOut:
+    // exp2(s c + ref) into the ring, and out of it (INTERIOR: the window of the chunk that Q = 0 completes is not
+    // the first or the last of its rows).  FILL: the wavefront requests one of its four pieces of the chunk three
+    // ahead (`fcbi` into `fstage`).  RAG: the quarter before has columns that do not exist (ragged last chunk):
+    // they stay out of sum and maximum.  All of these are compile-time flags: a branch inside the body would let
+    // the compiler move the arithmetic away from the matrix instructions it is threaded through.
+    auto quarter = [&](auto mode_c, auto q_c, auto mfma_c, auto fill_c, auto rag_c, auto int_c, int stage, int cprev,
+                       int fcbi, int fstage) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode_c)::value;
-        constexpr int hb = decltype(half_c)::value, pb = 1 - hb;
+        constexpr int Q = decltype(q_c)::value, PQ = (Q + 3) & 3, hb = Q & 1, pb = 1 - hb;
         constexpr bool MFMA = decltype(mfma_c)::value;
-        const unsigned char *sb = lds + stage * kRpStageBytes + 512 * hb;
-        const int colp = cprev * kRpCols + 4 * j + 2 * pb;     // first of the lane's two columns of the half before
-        float w[2];                                            // 0 for columns that do not exist (ragged last chunk)
-        w[0] = colp < N ? 1.f : 0.f;
-        w[1] = colp + 1 < N ? 1.f : 0.f;
-        unsigned char *wrow = ring + (4 * rg) * kRpRingPitch + ((cprev & 1) << 7) + (4 * j + 2 * pb) * 2;
-        u32x4 bf[2][2];
-        if constexpr (MFMA) {
-#pragma unroll
-            for (int ct = 0; ct < 2; ++ct) bf[0][ct] = *reinterpret_cast<const u32x4 *>(sb + boff0 + 256 * ct);
-        }
-        float xprev = 0.f, pprev = 0.f, plo = 0.f;
+        constexpr bool RAG = decltype(rag_c)::value;
+        constexpr bool INTERIOR = MODE == kRoleOut && decltype(int_c)::value;
+        const unsigned char *sb = lds + stage * kRpStageBytes + 4096 * Q;
+        const int b0 = rp_fresh(boff0);
+        const int colp = cprev * kRpCols + 16 * PQ + 4 * rg;       // the lane's columns of the quarter before: colp + i
+        // ring position of those columns; quarter 0 of a chunk in the first half of the ring also goes behind the
+        // row's end (pieces that start in a row's last 16 bytes continue there); in the second half the copy falls on
+        // the original
+        const int slot = (cprev & 1) << 7;
+        unsigned char *wrow = lds + rp_fresh(ringw_o) + slot + 32 * PQ;
+        unsigned char *wcopy = lds + rp_fresh(ringw_o) + 256 - slot;
+        u32x4 bf[2];
+        if constexpr (MFMA) bf[0] = *reinterpret_cast<const u32x4 *>(sb + b0);
+        float xprev = 0.f, pprev = 0.f, q0 = 0.f, q1 = 0.f, q2 = 0.f;
+        // element e of a quarter: row tile e / 4, column e % 4 of the lane's four
         auto use = [&](auto e_c, float pval) {
-            constexpr int pe = decltype(e_c)::value, prt = pe >> 3, pi = (pe >> 1) & 3, pct = pe & 1;
-            if constexpr (MODE == kRoleSum) sum[prt][pi] = fmaf(pval, w[pct], sum[prt][pi]);
-            else if constexpr (MODE == kRoleMax) sum[prt][pi] = __builtin_fmaxf(sum[prt][pi], w[pct] != 0.f ? pval : -3.0e38f);
-            else if constexpr (MODE == kRoleOut) {
-                if constexpr (pct == 0) plo = pval;
+            constexpr int pe = decltype(e_c)::value, prt = pe >> 2, pi = pe & 3;
+            if constexpr (MODE == kRoleSum) {
+                if constexpr (RAG) sum[prt] += colp + pi < N ? pval : 0.f;
+                else sum[prt] += pval;
+            } else if constexpr (MODE == kRoleMax) {
+                if constexpr (RAG) sum[prt] = __builtin_fmaxf(sum[prt], colp + pi < N ? pval : -3.0e38f);
+                else sum[prt] = __builtin_fmaxf(sum[prt], pval);
+            } else if constexpr (MODE == kRoleOut) {
+                if constexpr (pi == 0) q0 = pval;
+                else if constexpr (pi == 1) q1 = pval;
+                else if constexpr (pi == 2) q2 = pval;
                 else {
-                    *reinterpret_cast<uint32_t *>(wrow + (16 * prt + pi) * kRpRingPitch) = Elem<DT>::pack2(plo, pval);
-                    if constexpr (hb == 0 && (pe & 7) == 7)
-                        ring_store_rows(cprev, std::integral_constant<int, prt>{});   // the row tile is in the ring, both halves
+                    const u32x2 v = {Elem<DT>::pack2(q0, q1), Elem<DT>::pack2(q2, pval)};
+                    *reinterpret_cast<u32x2 *>(wrow + 16 * prt * kRpRingPitch) = v;
+                    if constexpr (PQ == 0) *reinterpret_cast<u32x2 *>(wcopy + 16 * prt * kRpRingPitch) = v;
+                }
+                // Out of the ring.  Quarter 3 of chunk cprev (done during Q = 0) completes the rows, row tile by row
+                // tile; row tile rt leaves as store instructions 2 rt and 2 rt + 1: load at its last element, store
+                // and load two elements on, store two further on; what is left of the last row tile rides in the
+                // first elements of Q = 1 (which writes those rows last).
+                if constexpr (INTERIOR && Q == 0 && (pe & 1) == 1) {
+                    constexpr int k = (pe - 3) / 2;            // steps: element 3 + 2k, k = 0 .. 6
+                    if constexpr (pe >= 3) {
+                        if constexpr (k % 2 == 0 && k >= 2) ring_store(cprev, std::integral_constant<int, k - 1>{});
+                        if constexpr (k % 2 == 1) ring_store(cprev, std::integral_constant<int, k - 1>{});
+                        ring_load(cprev, std::integral_constant<int, k>{});
+                    }
+                }
+                if constexpr (INTERIOR && Q == 1) {
+                    if constexpr (pe == 1) { ring_store(cprev - 1, std::integral_constant<int, 6>{}); ring_load(cprev - 1, std::integral_constant<int, 7>{}); }
+                    if constexpr (pe == 3) ring_store(cprev - 1, std::integral_constant<int, 7>{});
                 }
             }
         };
+#ifdef RP_X_NOEXP
+        auto power = [&](float x) { return x; };
+#else
         auto power = [&](float x) { return MODE == kRoleMax ? x : __builtin_amdgcn_exp2f(x); };
+#endif
         auto element = [&](auto e_c) {
-            constexpr int e = decltype(e_c)::value, rt2 = e >> 3, i2 = (e >> 1) & 3, ct2 = e & 1;
+            constexpr int e = decltype(e_c)::value, rt2 = e >> 2, i2 = e & 3;
             if constexpr (e >= 2) use(std::integral_constant<int, e - 2>{}, pprev);
             if constexpr (e >= 1) pprev = power(xprev);
-            const float sc = acc[pb][rt2][ct2][i2];
-            xprev = MODE == kRoleMax ? sc : fmaf(sc, c, ref[rt2][i2]);
+            const float sc = acc[pb][rt2][i2];
+            xprev = MODE == kRoleMax ? sc : fmaf(sc, c, ref[rt2]);
         };
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            if constexpr (MFMA) {
-                if (ks + 1 < 4) {
-#pragma unroll
-                    for (int ct = 0; ct < 2; ++ct)
-                        bf[(ks + 1) & 1][ct] = *reinterpret_cast<const u32x4 *>(sb + (boff0 ^ (64 * (ks + 1))) + 256 * ct);
-                }
+            if constexpr (decltype(fill_c)::value) {
+                if (ks == 2) fill_one(q_c, fcbi, fstage);
             }
-            auto group = [&](auto qd_c) {
-                constexpr int qd = decltype(qd_c)::value, rt = qd >> 1, ct = qd & 1;
+            if constexpr (MFMA) {
+                if (ks + 1 < 4) bf[(ks + 1) & 1] = *reinterpret_cast<const u32x4 *>(sb + (b0 ^ (64 * (ks + 1))));
+            }
+            auto group = [&](auto rt_c) {
+                constexpr int rt = decltype(rt_c)::value;
+                // (rows of B_g as the first operand: the lane gets row 16 rt + j, columns 4 rg .. 4 rg + 3 of the tile)
                 if constexpr (MFMA)
-                    acc[hb][rt][ct] = Elem<DT>::mfma(af[rt][ks], bf[ks & 1][ct],
-                                                     ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[hb][rt][ct]);
+                    acc[hb][rt] = Elem<DT>::mfma(bf[ks & 1], af[rt][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[hb][rt]);
                 if constexpr (MODE != 0) {
-                    if (ks == 0) element(std::integral_constant<int, 0 * 8 + qd>{});
-                    if (ks == 1) element(std::integral_constant<int, 1 * 8 + qd>{});
-                    if (ks == 2) element(std::integral_constant<int, 2 * 8 + qd>{});
-                    if (ks == 3) element(std::integral_constant<int, 3 * 8 + qd>{});
+                    if (ks == 0) element(std::integral_constant<int, 0 * 4 + rt>{});
+                    if (ks == 1) element(std::integral_constant<int, 1 * 4 + rt>{});
+                    if (ks == 2) element(std::integral_constant<int, 2 * 4 + rt>{});
+                    if (ks == 3) element(std::integral_constant<int, 3 * 4 + rt>{});
                 }
                 __builtin_amdgcn_sched_barrier(0);
             };
             group(I0{}); group(I1{}); group(I2{}); group(I3{});
-            group(std::integral_constant<int, 4>{}); group(std::integral_constant<int, 5>{});
-            group(std::integral_constant<int, 6>{}); group(std::integral_constant<int, 7>{});
         }
         if constexpr (MODE != 0) {
-            use(std::integral_constant<int, 30>{}, pprev);
+            use(std::integral_constant<int, 14>{}, pprev);
             pprev = power(xprev);
-            use(std::integral_constant<int, 31>{}, pprev);
+            use(std::integral_constant<int, 15>{}, pprev);
         }
     };
 
-    // sweep 1, first half chunk: the reference of every row = its maximum over these 32 columns
+    // sweep 1, first quarter chunk: the reference of every row = its maximum over these 16 columns (the lane's
+    // four, then the four lanes that share the row)
     auto stats_reference = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int rt = 0; rt < kRpRT; ++rt) {
-            float mx[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) mx[i] = __builtin_fmaxf(acc[0][rt][0][i], acc[0][rt][1][i]);
-            row16_max4(mx);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ref[rt][i] = -__builtin_fmaxf(mx[i], -3.0e38f) * c;
+            const float m = quad_column_max(__builtin_fmaxf(__builtin_fmaxf(acc[0][rt][0], acc[0][rt][1]),
+                                                            __builtin_fmaxf(acc[0][rt][2], acc[0][rt][3])));
+            ref[rt] = -__builtin_fmaxf(m, -3.0e38f) * c;
         }
     };
-    // after the last chunk of sweep 1: row sums over the sixteen lanes; returns whether any is not finite
+    // after the last chunk of sweep 1: row sums over the four lanes of a row; returns whether any is not finite
     auto finish_stats = [&]() __attribute__((always_inline)) {
         bool bad = false;
 #pragma unroll
         for (int rt = 0; rt < kRpRT; ++rt) {
-            float sm[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) sm[i] = sum[rt][i];
-            row16_sum4(sm);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                bad |= !(sm[i] <= 3.0e38f);
-                ref[rt][i] -= __builtin_amdgcn_logf(sm[i]);      // 1/sum goes into the exponent
-            }
+            const float sm = quad_column_sum(sum[rt]);
+            bad |= !(sm <= 3.0e38f);
+            ref[rt] -= __builtin_amdgcn_logf(sm);                // 1/sum goes into the exponent
         }
         return bad;
     };
     // after the maximum sweep: the reference of every row = its maximum over all columns
     auto finish_max = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int rt = 0; rt < kRpRT; ++rt) {
-            float mx[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) mx[i] = sum[rt][i];
-            row16_max4(mx);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ref[rt][i] = -__builtin_fmaxf(mx[i], -3.0e38f) * c;
-        }
+        for (int rt = 0; rt < kRpRT; ++rt) ref[rt] = -__builtin_fmaxf(quad_column_max(sum[rt]), -3.0e38f) * c;
     };
 
     // -------- the steps.  All of this is the same in every wavefront of the workgroup (scalar registers).
@@ -440,54 +464,97 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         if (first_step) {
             if (filler) {
                 for (int k = 0; k < kRpStages - 1; ++k) fill(k, k);
-                wait_vm<0>();
-            } else {
-                wait_vm<0>();                              // the A fragments
             }
+            wait_vm<0>();                                  // the first chunks, or the A fragments
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             first_step = false;
         }
         // SYNC of iteration i: the filling wavefronts wait for their part of chunk i (requested three iterations
-        // ago, right behind that iteration's barrier; the fills of the two iterations since may stay in flight;
-        // the first three chunks of a step were complete before the step began), barrier (now everyone's part is
-        // there and nobody reads the stage of chunk i - 1 any more), request chunk i + 3 -- which, in any step but
-        // the workgroup's last, is a chunk of the next step once the end of B_g is near.
-        auto sync = [&](int i) __attribute__((always_inline)) {
+        // ago; the fills of the two iterations since may stay in flight; the first three chunks of a step were
+        // complete before the step began), barrier (now everyone's part is there and nobody reads the stage of
+        // chunk i - 1 any more), request chunk i + 3 -- which, in any step but the workgroup's last, is a chunk of
+        // the next step once the end of B_g is near.  `spread`: the quarters of the iteration issue the four
+        // instructions of the request one by one instead (a load into LDS holds the wavefront that issues it while
+        // the requests before it are taken, about 70 cycles each, so four wavefronts issuing four in a row wait for
+        // each other).
+        int pf_cbi = 0, pf_stage = 0;
+        auto sync = [&](int i, bool spread) __attribute__((always_inline)) {
             if (filler && i >= kRpStages - 1) {
                 int later = 2 * kRpFillInsts;
                 if (final_step) later = kRpFillInsts * ((i + 1 < ncb ? 1 : 0) + (i + 2 < ncb ? 1 : 0));
                 rp_wait_vm_upto(later);
             }
+#ifdef RP_X_NOBAR
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#else
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            if (filler && (!final_step || i + kRpStages - 1 < ncb)) {
-                int cbi = i + kRpStages - 1;
-                if (cbi >= ncb) cbi -= ncb;
-                fill(cbi, (gpos + i + kRpStages - 1) & (kRpStages - 1));
-            }
+#endif
+            int cbi = i + kRpStages - 1;
+            if (cbi >= ncb) cbi -= ncb;
+            pf_cbi = cbi;
+            pf_stage = (gpos + i + kRpStages - 1) & (kRpStages - 1);
+            if (!spread && filler && (!final_step || i + kRpStages - 1 < ncb)) fill(pf_cbi, pf_stage);
             __builtin_amdgcn_sched_barrier(0);
         };
-        auto run = [&](auto mode_c) __attribute__((always_inline)) {
+        // FILL: the wavefront issues its fills from inside the quarters (it is this step's filler, the step is not
+        // the workgroup's last, so every iteration has a chunk to request, and K > 0).
+        auto run = [&](auto mode_c, auto fill_c) __attribute__((always_inline)) {
             constexpr int MODE = decltype(mode_c)::value;
-            using False = std::false_type;
-            using True = std::true_type;
+            using Fill = decltype(fill_c);
+            using Out = std::integral_constant<bool, MODE == kRoleOut>;
             // (a wavefront without rows only keeps the barriers and its fills: decided once, so that the accumulators
             // are plainly defined before they are used in the branch that computes)
             if (!active) {
-                for (int i = 0; i < ncb; ++i) sync(i);
+                for (int i = 0; i < ncb; ++i) sync(i, false);
                 return;
             }
-            sync(0);
-            half_body(I0{}, I0{}, True{}, gpos & (kRpStages - 1), 0);
-            if (MODE == kRoleSum && my_role == kRoleSum) stats_reference();
-            half_body(mode_c, I1{}, True{}, gpos & (kRpStages - 1), 0);
-            for (int i = 1; i < ncb; ++i) {
-                sync(i);
-                const int stage = (gpos + i) & (kRpStages - 1);
-                half_body(mode_c, I0{}, True{}, stage, i - 1);
-                if (MODE == kRoleOut && i == 1) ring_store_edge(0);
-                half_body(mode_c, I1{}, True{}, stage, i);
+            const bool ragged = (N & (kRpCols - 1)) != 0;
+            // chunk 0: nothing to do arithmetic on yet; sweep 1 takes its reference from the first quarter
+            {
+                const int stage = gpos & (kRpStages - 1);
+                sync(0, Fill::value);
+                quarter(I0{}, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                if (MODE == kRoleSum && my_role == kRoleSum) stats_reference();
+                quarter(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
             }
-            half_body(mode_c, I0{}, False{}, 0, ncb - 1);
+            // chunk 1: completes chunk 0, whose window is an edge
+            {
+                sync(1, Fill::value);
+                const int stage = (gpos + 1) & (kRpStages - 1);
+                quarter(mode_c, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                if (MODE == kRoleOut) ring_store_edge(0);
+                quarter(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
+                quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
+                quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
+            }
+            for (int i = 2; i < ncb - 1; ++i) {
+                sync(i, Fill::value);
+                const int stage = (gpos + i) & (kRpStages - 1);
+                quarter(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
+                quarter(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
+                quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
+                quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
+            }
+            // the last chunk: its columns may end early (sweep 1 and the maximum sweep leave the missing ones out)
+            {
+                const int i = ncb - 1;
+                sync(i, Fill::value);
+                const int stage = (gpos + i) & (kRpStages - 1);
+                quarter(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
+                if (MODE != kRoleOut && ragged) {
+                    quarter(mode_c, I1{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
+                    quarter(mode_c, I2{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
+                    quarter(mode_c, I3{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
+                    quarter(mode_c, I0{}, False{}, False{}, True{}, False{}, 0, i, 0, 0);
+                } else {
+                    quarter(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
+                    quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
+                    quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
+                    quarter(mode_c, I0{}, False{}, False{}, False{}, False{}, 0, i, 0, 0);
+                }
+            }
             if (MODE == kRoleOut) ring_store_edge(ncb - 1);
         };
         // Every role keeps its state inside its own branch: what a sweep sets up, it alone uses (the sums of sweep 1,
@@ -495,22 +562,19 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         volatile int *fl = flags + 2 * (step & 1);
         if (my_role == kRoleOut) {
             store_lanes();
-            run(std::integral_constant<int, kRoleOut>{});
+            run(std::integral_constant<int, kRoleOut>{}, False{});
         } else if (my_role == kRoleMax) {
 #pragma unroll
-            for (int rt = 0; rt < kRpRT; ++rt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) sum[rt][i] = -3.0e38f;
-            run(std::integral_constant<int, kRoleMax>{});
+            for (int rt = 0; rt < kRpRT; ++rt) sum[rt] = -3.0e38f;
+            run(std::integral_constant<int, kRoleMax>{}, False{});
             if (active) finish_max();
         } else if (my_role == kRoleNone) {
-            for (int i = 0; i < ncb; ++i) sync(i);
+            for (int i = 0; i < ncb; ++i) sync(i, false);
         } else {
 #pragma unroll
-            for (int rt = 0; rt < kRpRT; ++rt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) sum[rt][i] = 0.f;
-            run(std::integral_constant<int, kRoleSum>{});
+            for (int rt = 0; rt < kRpRT; ++rt) sum[rt] = 0.f;
+            if (filler && fills_on) run(std::integral_constant<int, kRoleSum>{}, True{});
+            else run(std::integral_constant<int, kRoleSum>{}, False{});
             // the overflow verdict of sweep 1 goes to the whole workgroup through LDS
             const bool bad = active && finish_stats();
             if (my_role == kRoleSum && __ballot(bad) != 0 && lane == 0) fl[set] = 1;
