@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     u32x4 af[kRpRT][4];                        // A fragments [rt][ks]: row 16 rt + j, k = 32 ks + 8 rg ..
     float ref[kRpRT];                          // of row 16 rt + j; sweep 1: -R c; sweep 2: -R c - log2(sum)
     float sum[kRpRT];                          // sweep 1: running sum over the lane's columns; maximum sweep: running maximum
-    f32x4 acc[2][kRpRT];                       // [quarter % 2][rt]: columns 4 rg + i of the quarter's column tile
+    f32x4 acc[2][kRpRT][2];                    // [half][rt][column tile of the half]: columns 4 rg + i of the tile
     uint32_t v0[kRpStoreInsts];                // sweep 2: byte offset of the lane's piece of window 0 inside the segment's result
     int upos[kRpStoreInsts];                   // ... and ring byte of that piece: 2 (8q - d) mod 256
     int row0 = 0;
@@ -306,42 +306,45 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     using False = std::false_type;
     using True = std::true_type;
 
-    // -------- one quarter: the 16 matrix instructions of column tile Q of the chunk in `stage` (when MFMA) into
-    // accumulator set Q % 2, with the arithmetic of the quarter before -- quarter (Q + 3) % 4 of chunk `cprev`, in
-    // the other accumulator set -- threaded between them, one score element per matrix instruction.
+    // -------- one half: the 32 matrix instructions of half HB (column tiles 2 HB, 2 HB + 1) of the chunk in `stage`
+    // (when MFMA) into accumulator set HB, with the arithmetic of the half before -- half 1 - HB of chunk `cprev`,
+    // in the other accumulator set -- threaded between them, one score element per matrix instruction.
     // MODE 0: matrix instructions only; kRoleSum: sum += exp2(s c + ref); kRoleMax: running maximum; kRoleOut:
-    // exp2(s c + ref) into the ring, and out of it (INTERIOR: the window of the chunk that Q = 0 completes is not
-    // the first or the last of its rows).  FILL: the wavefront requests one of its four pieces of the chunk three
-    // ahead (`fcbi` into `fstage`).  RAG: the quarter before has columns that do not exist (ragged last chunk):
-    // they stay out of sum and maximum.  All of these are compile-time flags: a branch inside the body would let
-    // the compiler move the arithmetic away from the matrix instructions it is threaded through.
-    auto quarter = [&](auto mode_c, auto q_c, auto mfma_c, auto fill_c, auto rag_c, auto int_c, int stage, int cprev,
-                       int fcbi, int fstage) __attribute__((always_inline)) {
+    // exp2(s c + ref) into the ring, and out of it (INTERIOR: the window of the chunk that HB = 0 completes is not
+    // the first or the last of its rows).  FILL: the wavefront requests two of its four pieces of the chunk three
+    // ahead (`fcbi` into `fstage`).  RAG: the half before has columns that do not exist (ragged last chunk): they
+    // stay out of sum and maximum.  All of these are compile-time flags: a branch inside the body would let the
+    // compiler move the arithmetic away from the matrix instructions it is threaded through.
+    auto half = [&](auto mode_c, auto h_c, auto mfma_c, auto fill_c, auto rag_c, auto int_c, int stage, int cprev,
+                    int fcbi, int fstage) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode_c)::value;
-        constexpr int Q = decltype(q_c)::value, PQ = (Q + 3) & 3, hb = Q & 1, pb = 1 - hb;
+        constexpr int hb = decltype(h_c)::value, pb = 1 - hb;
         constexpr bool MFMA = decltype(mfma_c)::value;
         constexpr bool RAG = decltype(rag_c)::value;
         constexpr bool INTERIOR = MODE == kRoleOut && decltype(int_c)::value;
-        const unsigned char *sb = lds + stage * kRpStageBytes + 4096 * Q;
+        const unsigned char *sb = lds + stage * kRpStageBytes + 8192 * hb;
         const int b0 = rp_fresh(boff0);
-        const int colp = cprev * kRpCols + 16 * PQ + 4 * rg;       // the lane's columns of the quarter before: colp + i
-        // ring position of those columns; quarter 0 of a chunk in the first half of the ring also goes behind the
-        // row's end (pieces that start in a row's last 16 bytes continue there); in the second half the copy falls on
-        // the original
+        const int colp = cprev * kRpCols + 32 * pb + 4 * rg;       // the lane's columns of the half before: colp + 16 ct + i
+        // ring position of those columns; the first column tile of a chunk in the first half of the ring also goes
+        // behind the row's end (pieces that start in a row's last 16 bytes continue there); in the second half the
+        // copy falls on the original
         const int slot = (cprev & 1) << 7;
-        unsigned char *wrow = lds + rp_fresh(ringw_o) + slot + 32 * PQ;
+        unsigned char *wrow = lds + rp_fresh(ringw_o) + slot + 64 * pb;
         unsigned char *wcopy = lds + rp_fresh(ringw_o) + 256 - slot;
-        u32x4 bf[2];
-        if constexpr (MFMA) bf[0] = *reinterpret_cast<const u32x4 *>(sb + b0);
+        u32x4 bf[2][2];
+        if constexpr (MFMA) {
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct) bf[0][ct] = *reinterpret_cast<const u32x4 *>(sb + b0 + 4096 * ct);
+        }
         float xprev = 0.f, pprev = 0.f, q0 = 0.f, q1 = 0.f, q2 = 0.f;
-        // element e of a quarter: row tile e / 4, column e % 4 of the lane's four
+        // element e of a half: row tile e / 8, column tile (e / 4) % 2, column e % 4 of the lane's four
         auto use = [&](auto e_c, float pval) {
-            constexpr int pe = decltype(e_c)::value, prt = pe >> 2, pi = pe & 3;
+            constexpr int pe = decltype(e_c)::value, prt = pe >> 3, pct = (pe >> 2) & 1, pi = pe & 3;
             if constexpr (MODE == kRoleSum) {
-                if constexpr (RAG) sum[prt] += colp + pi < N ? pval : 0.f;
+                if constexpr (RAG) sum[prt] += colp + 16 * pct + pi < N ? pval : 0.f;
                 else sum[prt] += pval;
             } else if constexpr (MODE == kRoleMax) {
-                if constexpr (RAG) sum[prt] = __builtin_fmaxf(sum[prt], colp + pi < N ? pval : -3.0e38f);
+                if constexpr (RAG) sum[prt] = __builtin_fmaxf(sum[prt], colp + 16 * pct + pi < N ? pval : -3.0e38f);
                 else sum[prt] = __builtin_fmaxf(sum[prt], pval);
             } else if constexpr (MODE == kRoleOut) {
                 if constexpr (pi == 0) q0 = pval;
@@ -349,24 +352,23 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
                 else if constexpr (pi == 2) q2 = pval;
                 else {
                     const u32x2 v = {Elem<DT>::pack2(q0, q1), Elem<DT>::pack2(q2, pval)};
-                    *reinterpret_cast<u32x2 *>(wrow + 16 * prt * kRpRingPitch) = v;
-                    if constexpr (PQ == 0) *reinterpret_cast<u32x2 *>(wcopy + 16 * prt * kRpRingPitch) = v;
+                    *reinterpret_cast<u32x2 *>(wrow + 16 * prt * kRpRingPitch + 32 * pct) = v;
+                    if constexpr (pb == 0 && pct == 0) *reinterpret_cast<u32x2 *>(wcopy + 16 * prt * kRpRingPitch) = v;
                 }
-                // Out of the ring.  Quarter 3 of chunk cprev (done during Q = 0) completes the rows, row tile by row
+                // Out of the ring.  Half 1 of chunk cprev (done during HB = 0) completes the rows, row tile by row
                 // tile; row tile rt leaves as store instructions 2 rt and 2 rt + 1: load at its last element, store
-                // and load two elements on, store two further on; what is left of the last row tile rides in the
-                // first elements of Q = 1 (which writes those rows last).
-                if constexpr (INTERIOR && Q == 0 && (pe & 1) == 1) {
-                    constexpr int k = (pe - 3) / 2;            // steps: element 3 + 2k, k = 0 .. 6
-                    if constexpr (pe >= 3) {
-                        if constexpr (k % 2 == 0 && k >= 2) ring_store(cprev, std::integral_constant<int, k - 1>{});
-                        if constexpr (k % 2 == 1) ring_store(cprev, std::integral_constant<int, k - 1>{});
+                // and load four elements on, store four further on; what is left of the last row tile rides in the
+                // first elements of HB = 1 (which writes those rows last).
+                if constexpr (INTERIOR && hb == 0 && (pe & 3) == 3) {
+                    constexpr int k = (pe - 7) / 4;            // steps at elements 7, 11, 15, .., 31: k = 0 .. 6
+                    if constexpr (pe >= 7) {
+                        if constexpr (k >= 1) ring_store(cprev, std::integral_constant<int, k - 1>{});
                         ring_load(cprev, std::integral_constant<int, k>{});
                     }
                 }
-                if constexpr (INTERIOR && Q == 1) {
-                    if constexpr (pe == 1) { ring_store(cprev - 1, std::integral_constant<int, 6>{}); ring_load(cprev - 1, std::integral_constant<int, 7>{}); }
-                    if constexpr (pe == 3) ring_store(cprev - 1, std::integral_constant<int, 7>{});
+                if constexpr (INTERIOR && hb == 1) {
+                    if constexpr (pe == 3) { ring_store(cprev - 1, std::integral_constant<int, 6>{}); ring_load(cprev - 1, std::integral_constant<int, 7>{}); }
+                    if constexpr (pe == 7) ring_store(cprev - 1, std::integral_constant<int, 7>{});
                 }
             }
         };
@@ -376,50 +378,58 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         auto power = [&](float x) { return MODE == kRoleMax ? x : __builtin_amdgcn_exp2f(x); };
 #endif
         auto element = [&](auto e_c) {
-            constexpr int e = decltype(e_c)::value, rt2 = e >> 2, i2 = e & 3;
+            constexpr int e = decltype(e_c)::value, rt2 = e >> 3, ct2 = (e >> 2) & 1, i2 = e & 3;
             if constexpr (e >= 2) use(std::integral_constant<int, e - 2>{}, pprev);
             if constexpr (e >= 1) pprev = power(xprev);
-            const float sc = acc[pb][rt2][i2];
+            const float sc = acc[pb][rt2][ct2][i2];
             xprev = MODE == kRoleMax ? sc : fmaf(sc, c, ref[rt2]);
         };
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             if constexpr (decltype(fill_c)::value) {
-                if (ks == 2) fill_one(q_c, fcbi, fstage);
+                if (ks == 1) fill_one(std::integral_constant<int, 2 * hb>{}, fcbi, fstage);
+                if (ks == 3) fill_one(std::integral_constant<int, 2 * hb + 1>{}, fcbi, fstage);
             }
             if constexpr (MFMA) {
-                if (ks + 1 < 4) bf[(ks + 1) & 1] = *reinterpret_cast<const u32x4 *>(sb + (b0 ^ (64 * (ks + 1))));
+                if (ks + 1 < 4) {
+#pragma unroll
+                    for (int ct = 0; ct < 2; ++ct)
+                        bf[(ks + 1) & 1][ct] = *reinterpret_cast<const u32x4 *>(sb + (b0 ^ (64 * (ks + 1))) + 4096 * ct);
+                }
             }
-            auto group = [&](auto rt_c) {
-                constexpr int rt = decltype(rt_c)::value;
+            auto group = [&](auto qd_c) {
+                constexpr int qd = decltype(qd_c)::value, rt = qd >> 1, ct = qd & 1;
                 // (rows of B_g as the first operand: the lane gets row 16 rt + j, columns 4 rg .. 4 rg + 3 of the tile)
                 if constexpr (MFMA)
-                    acc[hb][rt] = Elem<DT>::mfma(bf[ks & 1], af[rt][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[hb][rt]);
+                    acc[hb][rt][ct] = Elem<DT>::mfma(bf[ks & 1][ct], af[rt][ks],
+                                                     ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[hb][rt][ct]);
                 if constexpr (MODE != 0) {
-                    if (ks == 0) element(std::integral_constant<int, 0 * 4 + rt>{});
-                    if (ks == 1) element(std::integral_constant<int, 1 * 4 + rt>{});
-                    if (ks == 2) element(std::integral_constant<int, 2 * 4 + rt>{});
-                    if (ks == 3) element(std::integral_constant<int, 3 * 4 + rt>{});
+                    if (ks == 0) element(std::integral_constant<int, 0 * 8 + qd>{});
+                    if (ks == 1) element(std::integral_constant<int, 1 * 8 + qd>{});
+                    if (ks == 2) element(std::integral_constant<int, 2 * 8 + qd>{});
+                    if (ks == 3) element(std::integral_constant<int, 3 * 8 + qd>{});
                 }
                 __builtin_amdgcn_sched_barrier(0);
             };
             group(I0{}); group(I1{}); group(I2{}); group(I3{});
+            group(std::integral_constant<int, 4>{}); group(std::integral_constant<int, 5>{});
+            group(std::integral_constant<int, 6>{}); group(std::integral_constant<int, 7>{});
         }
         if constexpr (MODE != 0) {
-            use(std::integral_constant<int, 14>{}, pprev);
+            use(std::integral_constant<int, 30>{}, pprev);
             pprev = power(xprev);
-            use(std::integral_constant<int, 15>{}, pprev);
+            use(std::integral_constant<int, 31>{}, pprev);
         }
     };
 
-    // sweep 1, first quarter chunk: the reference of every row = its maximum over these 16 columns (the lane's
-    // four, then the four lanes that share the row)
+    // sweep 1, first half chunk: the reference of every row = its maximum over these 32 columns (the lane's
+    // eight, then the four lanes that share the row)
     auto stats_reference = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int rt = 0; rt < kRpRT; ++rt) {
-            const float m = quad_column_max(__builtin_fmaxf(__builtin_fmaxf(acc[0][rt][0], acc[0][rt][1]),
-                                                            __builtin_fmaxf(acc[0][rt][2], acc[0][rt][3])));
-            ref[rt] = -__builtin_fmaxf(m, -3.0e38f) * c;
+            float m = __builtin_fmaxf(__builtin_fmaxf(acc[0][rt][0][0], acc[0][rt][0][1]), __builtin_fmaxf(acc[0][rt][0][2], acc[0][rt][0][3]));
+            m = __builtin_fmaxf(m, __builtin_fmaxf(__builtin_fmaxf(acc[0][rt][1][0], acc[0][rt][1][1]), __builtin_fmaxf(acc[0][rt][1][2], acc[0][rt][1][3])));
+            ref[rt] = -__builtin_fmaxf(quad_column_max(m), -3.0e38f) * c;
         }
     };
     // after the last chunk of sweep 1: row sums over the four lanes of a row; returns whether any is not finite
@@ -473,7 +483,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         // ago; the fills of the two iterations since may stay in flight; the first three chunks of a step were
         // complete before the step began), barrier (now everyone's part is there and nobody reads the stage of
         // chunk i - 1 any more), request chunk i + 3 -- which, in any step but the workgroup's last, is a chunk of
-        // the next step once the end of B_g is near.  `spread`: the quarters of the iteration issue the four
+        // the next step once the end of B_g is near.  `spread`: the halves of the iteration issue the four
         // instructions of the request one by one instead (a load into LDS holds the wavefront that issues it while
         // the requests before it are taken, about 70 cycles each, so four wavefronts issuing four in a row wait for
         // each other).
@@ -482,7 +492,9 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             if (filler && i >= kRpStages - 1) {
                 int later = 2 * kRpFillInsts;
                 if (final_step) later = kRpFillInsts * ((i + 1 < ncb ? 1 : 0) + (i + 2 < ncb ? 1 : 0));
+#ifndef RP_X_NOWAIT
                 rp_wait_vm_upto(later);
+#endif
             }
 #ifdef RP_X_NOBAR
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -496,7 +508,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             if (!spread && filler && (!final_step || i + kRpStages - 1 < ncb)) fill(pf_cbi, pf_stage);
             __builtin_amdgcn_sched_barrier(0);
         };
-        // FILL: the wavefront issues its fills from inside the quarters (it is this step's filler, the step is not
+        // FILL: the wavefront issues its fills from inside the halves (it is this step's filler, the step is not
         // the workgroup's last, so every iteration has a chunk to request, and K > 0).
         auto run = [&](auto mode_c, auto fill_c) __attribute__((always_inline)) {
             constexpr int MODE = decltype(mode_c)::value;
@@ -509,50 +521,40 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
                 return;
             }
             const bool ragged = (N & (kRpCols - 1)) != 0;
-            // chunk 0: nothing to do arithmetic on yet; sweep 1 takes its reference from the first quarter
+            // chunk 0: nothing to do arithmetic on yet; sweep 1 takes its reference from the first half
             {
                 const int stage = gpos & (kRpStages - 1);
                 sync(0, Fill::value);
-                quarter(I0{}, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                half(I0{}, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
                 if (MODE == kRoleSum && my_role == kRoleSum) stats_reference();
-                quarter(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
-                quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
-                quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                half(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
             }
             // chunk 1: completes chunk 0, whose window is an edge
             {
                 sync(1, Fill::value);
                 const int stage = (gpos + 1) & (kRpStages - 1);
-                quarter(mode_c, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
+                half(mode_c, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
                 if (MODE == kRoleOut) ring_store_edge(0);
-                quarter(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
-                quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
-                quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
+                half(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
             }
             for (int i = 2; i < ncb - 1; ++i) {
                 sync(i, Fill::value);
                 const int stage = (gpos + i) & (kRpStages - 1);
-                quarter(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
-                quarter(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
-                quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
-                quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
+                half(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
+                half(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
             }
             // the last chunk: its columns may end early (sweep 1 and the maximum sweep leave the missing ones out)
             {
                 const int i = ncb - 1;
                 sync(i, Fill::value);
                 const int stage = (gpos + i) & (kRpStages - 1);
-                quarter(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
+                half(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
                 if (MODE != kRoleOut && ragged) {
-                    quarter(mode_c, I1{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
-                    quarter(mode_c, I2{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
-                    quarter(mode_c, I3{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
-                    quarter(mode_c, I0{}, False{}, False{}, True{}, False{}, 0, i, 0, 0);
+                    half(mode_c, I1{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);
+                    half(mode_c, I0{}, False{}, False{}, True{}, False{}, 0, i, 0, 0);
                 } else {
-                    quarter(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
-                    quarter(mode_c, I2{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
-                    quarter(mode_c, I3{}, True{}, Fill{}, False{}, False{}, stage, i, pf_cbi, pf_stage);
-                    quarter(mode_c, I0{}, False{}, False{}, False{}, False{}, 0, i, 0, 0);
+                    half(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
+                    half(mode_c, I0{}, False{}, False{}, False{}, False{}, 0, i, 0, 0);
                 }
             }
             if (MODE == kRoleOut) ring_store_edge(ncb - 1);
