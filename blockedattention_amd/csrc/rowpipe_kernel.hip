@@ -65,11 +65,15 @@ __device__ __forceinline__ void rp_wait_vm_upto(int n) {  // n in {0, 4, 8}, wav
     else wait_vm<0>();
 }
 
-// Sixteen bytes of a ring row starting at byte `pos` (any even value below 256): one LDS read at a 2-byte
-// alignment (the LDS takes wide accesses at any alignment; eight lanes reading eight consecutive pieces of a
-// row touch every bank once).
+// Sixteen bytes of a ring row starting at byte `pos` (any even value below 256): five aligned words, shifted.
+// (One 16-byte LDS read at that address works, but any LDS read wider than its alignment holds the LDS for about
+// 57 cycles per wavefront against 8 for an aligned one; five word reads of rows 74 words apart take about 18.)
 __device__ __forceinline__ u32x4 rp_ring_read16(const unsigned char *row, int pos) {
-    return *reinterpret_cast<const u32x4_unaligned *>(row + pos);
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(row + (pos & ~3));
+    const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
+    const uint32_t sh = (uint32_t)(pos & 2) * 8;
+    return u32x4{__builtin_amdgcn_alignbit(d1, d0, sh), __builtin_amdgcn_alignbit(d2, d1, sh),
+                 __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh)};
 }
 
 // A copy of a per-lane constant that the compiler cannot see through: what is derived from it inside a loop is
@@ -78,12 +82,6 @@ template <typename T> __device__ __forceinline__ T rp_fresh(T v) {
     asm volatile("" : "+v"(v));
     return v;
 }
-
-#ifdef RP_X_NOSTORE
-#define RP_STORE(v, res, off) do { u32x4 v_ = (v); uint32_t o_ = (off); asm volatile("" :: "v"(v_), "v"(o_)); } while (0)
-#else
-#define RP_STORE(v, res, off) __builtin_amdgcn_raw_buffer_store_b128(v, res, off, 0, 0)
-#endif
 
 template <int DT>
 __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int zdim, int weave) {
@@ -185,13 +183,11 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         // (the row clamp changes nothing in a whole chunk: two instructions, no branch)
         const int r = min(4 * i + (lane >> 4), N - 1 - cb);
         const uint32_t off = rp_fresh(fill_row) + (uint32_t)((r - 4 * wq - (lane >> 4)) * K) * 2u;
-#ifndef RP_X_NOFILL
         uint64_t saved;
         const uint64_t mask = fill_mask;
         asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
                      "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
                      : "=&s"(saved) : "v"(off), "s"(base), "s"(dst), "s"(mask) : "memory", "m0");
-#endif
     };
     auto fill = [&](int cbi, int stage) __attribute__((always_inline)) {
         if (!fills_on) return;
@@ -207,6 +203,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     float ref[kRpRT];                          // of row 16 rt + j; sweep 1: -R c; sweep 2: -R c - log2(sum)
     float sum[kRpRT];                          // sweep 1: running sum over the lane's columns; maximum sweep: running maximum
     f32x4 acc[2][kRpRT][2];                    // [half][rt][column tile of the half]: columns 4 rg + i of the tile
+    u32x4 bf[3][2];                            // B fragments of three k-steps: [buffer][column tile of the half]
     uint32_t v0[kRpStoreInsts];                // sweep 2: byte offset of the lane's piece of window 0 inside the segment's result
     int upos[kRpStoreInsts];                   // ... and ring byte of that piece: 2 (8q - d) mod 256
     int row0 = 0;
@@ -260,7 +257,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     };
     auto ring_store = [&](int cbi, auto t_c) __attribute__((always_inline)) {
         constexpr int t = decltype(t_c)::value;
-        RP_STORE(ring_ld, out_res, v0[t] + 128u * (uint32_t)cbi);        // (the range check sees the vector offset only)
+        __builtin_amdgcn_raw_buffer_store_b128(ring_ld, out_res, v0[t] + 128u * (uint32_t)cbi, 0, 0);        // (the range check sees the vector offset only)
         asm volatile("" ::: "memory");
     };
     // First or last chunk: pieces before column 0 or past column N are dropped, and the end pieces the windows
@@ -277,11 +274,11 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             const u32x4 v = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ par);
             const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRpCols * cbi;      // first column of the piece
             const uint32_t voff = (col < 0 || col + 8 > N) ? kRpOutOfRange : v0[t] + adv;
-            RP_STORE(v, out_res, voff);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
         }
         if (cbi == 0) {
             const u32x4 v = rp_ring_read16(et_base, 0);                         // columns [0, 8)
-            RP_STORE(v, out_res, et_off);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, 0);
         }
         if (cbi == ncb - 1) {
             // the window behind the last chunk (what is left of the rows), then columns [N-8, N)
@@ -291,10 +288,10 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
                 const u32x4 v = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ par2);
                 const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRpCols * ncb;
                 const uint32_t voff = col + 8 <= N ? v0[t] + 128u * (uint32_t)ncb : kRpOutOfRange;
-                RP_STORE(v, out_res, voff);
+                __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
             }
             const u32x4 v = rp_ring_read16(et_base, (2 * (N - 8)) & 255);
-            RP_STORE(v, out_res, et_off + 2u * (uint32_t)(N - 8));
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off + 2u * (uint32_t)(N - 8), 0, 0);
         }
         asm volatile("" ::: "memory");
     };
@@ -331,11 +328,16 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         const int slot = (cprev & 1) << 7;
         unsigned char *wrow = lds + rp_fresh(ringw_o) + slot + 64 * pb;
         unsigned char *wcopy = lds + rp_fresh(ringw_o) + 256 - slot;
-        u32x4 bf[2][2];
-        if constexpr (MFMA) {
-#pragma unroll
-            for (int ct = 0; ct < 2; ++ct) bf[0][ct] = *reinterpret_cast<const u32x4 *>(sb + b0 + 4096 * ct);
-        }
+        // B fragments: three buffers in rotation over the eight k-steps of a chunk (buffer (4 HB + ks) % 3), read two
+        // k-steps -- sixteen matrix instructions -- ahead; half 0 starts with the reads of its first two k-steps (the
+        // chunk is only known to be there after the barrier), half 1 finds its first two under way
+        auto bread = [&](auto g_c) __attribute__((always_inline)) {
+            constexpr int g = decltype(g_c)::value, gh = g >> 2, gk = g & 3;
+            const unsigned char *gb = lds + stage * kRpStageBytes + 8192 * gh + (b0 ^ (64 * gk));
+            bf[g % 3][0] = *reinterpret_cast<const u32x4 *>(gb);
+            bf[g % 3][1] = *reinterpret_cast<const u32x4 *>(gb + 4096);
+        };
+        if constexpr (MFMA && hb == 0) { bread(std::integral_constant<int, 0>{}); bread(std::integral_constant<int, 1>{}); }
         float xprev = 0.f, pprev = 0.f, q0 = 0.f, q1 = 0.f, q2 = 0.f;
         // element e of a half: row tile e / 8, column tile (e / 4) % 2, column e % 4 of the lane's four
         auto use = [&](auto e_c, float pval) {
@@ -356,27 +358,31 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
                     if constexpr (pb == 0 && pct == 0) *reinterpret_cast<u32x2 *>(wcopy + 16 * prt * kRpRingPitch) = v;
                 }
                 // Out of the ring.  Half 1 of chunk cprev (done during HB = 0) completes the rows, row tile by row
-                // tile; row tile rt leaves as store instructions 2 rt and 2 rt + 1: load at its last element, store
-                // and load four elements on, store four further on; what is left of the last row tile rides in the
-                // first elements of HB = 1 (which writes those rows last).
-                if constexpr (INTERIOR && hb == 0 && (pe & 3) == 3) {
-                    constexpr int k = (pe - 7) / 4;            // steps at elements 7, 11, 15, .., 31: k = 0 .. 6
-                    if constexpr (pe >= 7) {
-                        if constexpr (k >= 1) ring_store(cprev, std::integral_constant<int, k - 1>{});
-                        ring_load(cprev, std::integral_constant<int, k>{});
-                    }
+                // tile (row tile rt at element 8 rt + 7), and row tile rt leaves as store instructions 2 rt and
+                // 2 rt + 1.  The eight stores of a chunk are spread over both halves, one every eight matrix
+                // instructions, each four elements behind its LDS read -- a wavefront that issues its stores in a
+                // burst waits for the memory pipeline to take them.  Every read comes after the rows are complete and
+                // before HB = 1 writes the next chunk into them (row tile rt from element 8 rt on).
+                if constexpr (INTERIOR && hb == 0) {
+                    if constexpr (pe == 7) ring_load(cprev, std::integral_constant<int, 0>{});
+                    if constexpr (pe == 11) ring_store(cprev, std::integral_constant<int, 0>{});
+                    if constexpr (pe == 15) ring_load(cprev, std::integral_constant<int, 1>{});
+                    if constexpr (pe == 19) ring_store(cprev, std::integral_constant<int, 1>{});
+                    if constexpr (pe == 23) ring_load(cprev, std::integral_constant<int, 2>{});
+                    if constexpr (pe == 27) ring_store(cprev, std::integral_constant<int, 2>{});
+                    if constexpr (pe == 31) ring_load(cprev, std::integral_constant<int, 3>{});
                 }
                 if constexpr (INTERIOR && hb == 1) {
-                    if constexpr (pe == 3) { ring_store(cprev - 1, std::integral_constant<int, 6>{}); ring_load(cprev - 1, std::integral_constant<int, 7>{}); }
-                    if constexpr (pe == 7) ring_store(cprev - 1, std::integral_constant<int, 7>{});
+                    if constexpr (pe == 3) { ring_store(cprev - 1, std::integral_constant<int, 3>{}); ring_load(cprev - 1, std::integral_constant<int, 4>{}); }
+                    if constexpr (pe == 7) ring_store(cprev - 1, std::integral_constant<int, 4>{});
+                    if constexpr (pe == 11) ring_load(cprev - 1, std::integral_constant<int, 5>{});
+                    if constexpr (pe == 15) { ring_store(cprev - 1, std::integral_constant<int, 5>{}); ring_load(cprev - 1, std::integral_constant<int, 6>{}); }
+                    if constexpr (pe == 19) { ring_store(cprev - 1, std::integral_constant<int, 6>{}); ring_load(cprev - 1, std::integral_constant<int, 7>{}); }
+                    if constexpr (pe == 23) ring_store(cprev - 1, std::integral_constant<int, 7>{});
                 }
             }
         };
-#ifdef RP_X_NOEXP
-        auto power = [&](float x) { return x; };
-#else
         auto power = [&](float x) { return MODE == kRoleMax ? x : __builtin_amdgcn_exp2f(x); };
-#endif
         auto element = [&](auto e_c) {
             constexpr int e = decltype(e_c)::value, rt2 = e >> 3, ct2 = (e >> 2) & 1, i2 = e & 3;
             if constexpr (e >= 2) use(std::integral_constant<int, e - 2>{}, pprev);
@@ -391,17 +397,16 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
                 if (ks == 3) fill_one(std::integral_constant<int, 2 * hb + 1>{}, fcbi, fstage);
             }
             if constexpr (MFMA) {
-                if (ks + 1 < 4) {
-#pragma unroll
-                    for (int ct = 0; ct < 2; ++ct)
-                        bf[(ks + 1) & 1][ct] = *reinterpret_cast<const u32x4 *>(sb + (b0 ^ (64 * (ks + 1))) + 4096 * ct);
-                }
+                if (ks == 0 && 4 * hb + 2 < 8) bread(std::integral_constant<int, (4 * hb + 2) & 7>{});
+                if (ks == 1 && 4 * hb + 3 < 8) bread(std::integral_constant<int, (4 * hb + 3) & 7>{});
+                if (ks == 2 && 4 * hb + 4 < 8) bread(std::integral_constant<int, (4 * hb + 4) & 7>{});
+                if (ks == 3 && 4 * hb + 5 < 8) bread(std::integral_constant<int, (4 * hb + 5) & 7>{});
             }
             auto group = [&](auto qd_c) {
                 constexpr int qd = decltype(qd_c)::value, rt = qd >> 1, ct = qd & 1;
                 // (rows of B_g as the first operand: the lane gets row 16 rt + j, columns 4 rg .. 4 rg + 3 of the tile)
                 if constexpr (MFMA)
-                    acc[hb][rt][ct] = Elem<DT>::mfma(bf[ks & 1][ct], af[rt][ks],
+                    acc[hb][rt][ct] = Elem<DT>::mfma(bf[(4 * hb + ks) % 3][ct], af[rt][ks],
                                                      ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[hb][rt][ct]);
                 if constexpr (MODE != 0) {
                     if (ks == 0) element(std::integral_constant<int, 0 * 8 + qd>{});
@@ -492,15 +497,9 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             if (filler && i >= kRpStages - 1) {
                 int later = 2 * kRpFillInsts;
                 if (final_step) later = kRpFillInsts * ((i + 1 < ncb ? 1 : 0) + (i + 2 < ncb ? 1 : 0));
-#ifndef RP_X_NOWAIT
                 rp_wait_vm_upto(later);
-#endif
             }
-#ifdef RP_X_NOBAR
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#else
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#endif
             int cbi = i + kRpStages - 1;
             if (cbi >= ncb) cbi -= ncb;
             pf_cbi = cbi;
@@ -562,6 +561,9 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         // Every role keeps its state inside its own branch: what a sweep sets up, it alone uses (the sums of sweep 1,
         // the store lanes of sweep 2), so none of it occupies registers in the other sweeps.
         volatile int *fl = flags + 2 * (step & 1);
+        // the set that stores has more to do per chunk than the other: its wavefronts go first where both can issue
+        if (my_role == kRoleOut) __builtin_amdgcn_s_setprio(3);
+        else __builtin_amdgcn_s_setprio(0);
         if (my_role == kRoleOut) {
             store_lanes();
             run(std::integral_constant<int, kRoleOut>{}, False{});
@@ -615,9 +617,15 @@ int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_
     int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
     static const int forced_z = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE_Z"); return e ? atoi(e) : 0; }();
     static const int forced_w = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE_WEAVE"); return e ? atoi(e) : 0; }();
-    const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRpBlockRows - 1) / kRpBlockRows));
+    // Workgroups per pair Z: workgroup z takes the z-th share of the pair's row blocks, one after the other.  A share
+    // of n row blocks takes n + 1 steps, the first and the last with one set idle, so few large shares are better
+    // than many small ones -- but a share longer than the chip's mean load per compute unit is the last to finish.
+    // Measured on 16 x 16 pairs of 5 .. 16 row blocks: Z = 1 imbalance, Z = 2 1594 us, Z = 3 1649 us; one workgroup
+    // per compute unit with an equal share of all the work (contiguous runs of pairs and row blocks): 1744 .. 1906 us,
+    // the dies with the narrow pairs finishing last.  BLOCKEDATTN_ROWPIPE_Z and _WEAVE override.
     const int cus = device_cu_count();
-    int64_t z = std::min<int64_t>(z_max, std::max<int64_t>(1, (3 * (int64_t)cus + pairs - 1) / pairs));
+    const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRpBlockRows - 1) / kRpBlockRows));
+    int64_t z = std::min<int64_t>(z_max, std::max<int64_t>(1, (2 * (int64_t)cus + pairs - 1) / pairs));
     if (forced_z > 0) z = std::min<int64_t>(z_max, forced_z);
     const int64_t weave = std::max<int64_t>(1, std::min<int64_t>(forced_w > 0 ? forced_w : 1, pairs / kDies));
     pairs = (pairs / kDies + weave - 1) / weave * weave * kDies;       // whole turns
