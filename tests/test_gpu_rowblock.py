@@ -1,6 +1,7 @@
-"""Large segments with K <= 128 (the row-block kernel: 256 rows per workgroup, 64 columns at a time, results
-through an LDS ring into line-aligned stores) against the oracle: every line phase, ragged rows and columns,
-every reduction length, the overflow path of the first sweep, GEMM alone and fused."""
+"""Large segments with K <= 128 (the row-block kernels: 256 rows per workgroup or per wavefront set, 64 columns at
+a time, results through an LDS ring into line-aligned stores; the fused pair runs the two sweeps of adjacent row
+blocks side by side on one stream of B_g) against the oracle: every line phase, ragged rows and columns, every
+reduction length, the overflow path of the first sweep, GEMM alone and fused."""
 import numpy as np
 import pytest
 import torch
@@ -16,8 +17,9 @@ pytestmark = pytest.mark.gpu
 def test_shapes_and_phases(dev, dtype):
     # odd and even widths (rows then start at every 2-byte phase of a 128-byte line), widths around the chunk
     # and ring sizes, heights around the workgroup's 256 rows and a wavefront's 32, one row, K from 8 to 128
-    M = [300, 256, 257, 1, 40, 33, 513, 31]; N = [257, 300, 1000, 5000, 320, 321, 263, 384]
-    K = [64, 128, 8, 40, 96, 104, 120, 32]
+    # (and K = 0: no operand bytes at all, zeros for the product and 1/N for the fused pair)
+    M = [300, 256, 257, 1, 40, 33, 513, 31, 40]; N = [257, 300, 1000, 5000, 320, 321, 263, 384, 300]
+    K = [64, 128, 8, 40, 96, 104, 120, 32, 0]
     plan = run_all(dev, M, N, K, 3, dtype, 0.11, seed=7)
     assert plan.info.list_tile == len(M)
 
@@ -51,6 +53,30 @@ def test_scores_far_above_the_first_chunk(dev):
     ref = oracle.per_segment_torch(A, B, M, N, K, 1.0)
     assert_probs_close(out, ref, "overflow path")
     assert float(out[:, :100 * 700].float().max()) > 0.05     # sharply peaked rows, as constructed
+    assert plan.read().run_errors == 0
+
+
+def test_overflow_in_the_middle_of_a_run_of_row_blocks(dev):
+    # Seven row blocks of one segment go through a workgroup's two wavefront sets, one sweep apart.  Only rows of the
+    # fourth block overflow the first sweep: that set repeats its block in two safe sweeps while the other set waits
+    # where it must, and the blocks before and after take the ordinary path.  A second head keeps both orders of
+    # the sets in play (its shares of row blocks start at another parity).
+    M = np.array([1700]); N = np.array([900]); K = np.array([64])
+    A, B = random_operands(M, N, K, 2, torch.float16, seed=13)
+    A = A.abs() * 0.5 + 0.5; B = B.abs()
+    Bs = B.reshape(2, 900, 64)
+    Bs[:, :64] *= 0.01                                        # tiny scores in the first chunk
+    As = A.reshape(2, 1700, 64)
+    As[:, :768] *= 0.02; As[:, 1024:] *= 0.02                 # only rows 768 .. 1023 reach far above it
+    Bs[:, 500:520] *= 6
+    plan = make_plan(dev, M, N, K)
+    i = plan.info
+    out = torch.full((2, i.Dout), float("nan"), dtype=torch.float16, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, 2, i.Dm1, i.Dm2, i.Dout, 1.0)
+    ref = oracle.per_segment_torch(A, B, M, N, K, 1.0)
+    assert_probs_close(out, ref, "overflow in one row block of seven")
+    peaked = out[:, 768 * 900:1024 * 900].float().max()
+    assert float(peaked) > 0.04                               # sharply peaked rows, as constructed
     assert plan.read().run_errors == 0
 
 
