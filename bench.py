@@ -53,7 +53,7 @@ def measured_traffic(workload, kernel):
 
 # the fused kernel that carries each configuration (its name in a rocprofv3 kernel trace)
 DOMINANT_KERNEL = {1: "ba::strip_kernel", 2: "ba::strip_kernel", 3: "ba::strip_kernel", 4: "ba::strip_kernel",
-                   5: "ba::rowblock_kernel"}
+                   5: "ba::rowpipe_kernel"}
 
 
 def parse():

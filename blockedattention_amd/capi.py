@@ -18,7 +18,7 @@ META_FROM_LISTS, META_FROM_ACCUM, META_GIVEN = 0, 1, 2
 SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
     "ba_plan_read_into", "ba_plan_gemm_notify", "ba_plan_softmax_notify", "ba_plan_wait",
-    "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax", "ba_repack_operand",
+    "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax",
     "ba_varlen_attention", "ba_gemm_softmax_static",
 )
 MAILBOX_BYTES = 320
@@ -87,8 +87,6 @@ def load():
     lib.ba_blocked_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, i64, i64, f32, vp]
     lib.ba_blocked_softmax_backward.restype = i32
     lib.ba_blocked_softmax_backward.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i64, i64, f32, vp]
-    lib.ba_repack_operand.restype = i32
-    lib.ba_repack_operand.argtypes = [vp, i32, i32, i32, vp, i32, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, i64, i64, i64, vp]
     lib.ba_gemm_softmax.restype = i32
     lib.ba_gemm_softmax.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
     lib.ba_varlen_attention.restype = i32
@@ -262,13 +260,3 @@ def varlen_attention(plan, Q, K, V, out, H, Dm1, Dm2, Dout, scale=1.0):
                                     _ptr(out), H, Dm1, Dm2, Dout, float(scale), _stream())
     check(st, "ba_varlen_attention")
     return out
-
-
-def repack_operand(src_plan, src_which, dst_plan, dst_which, src, dst, H, Dsrc, Ddst, swap_dims=False,
-                   column_major=False):
-    """dst operand ``dst_which`` of ``dst_plan`` <- operand ``src_which`` of ``src_plan`` (see ba_repack_operand)."""
-    st = load().ba_repack_operand(src_plan.ptr, src_which, int(swap_dims), int(column_major), dst_plan.ptr, dst_which,
-                                  dst_plan._hint(), src_plan.nseg, dtype_code(src.dtype), _ptr(src), _ptr(dst), H, Dsrc,
-                                  Ddst, _stream())
-    check(st, "ba_repack_operand")
-    return dst

@@ -69,11 +69,6 @@ int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *d
 int launch_softmax_backward(int dtype, void *plan, int64_t nseg, const void *y, const void *dy, void *dx, int64_t H,
                             int64_t Dsrc, float scale, const ba_plan_info *info, hipStream_t stream);
 
-// One operand of every segment copied (or transposed) into zero-padded row-major rows (see repack.hip).
-int launch_repack(const void *src_plan, int src_which, int swap_dims, int column_major, const void *dst_plan,
-                  int dst_which, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc, int64_t Ddst,
-                  const ba_plan_info *dst_info, hipStream_t stream);
-
 // Varlen attention O = softmax(scale Q K^T) V without the probabilities in memory (see attention.hip).
 // args.A = Q, args.B = K, args.out = O ([H, Dm1]); V has K's layout.
 int launch_attention(int dtype, const RunArgs &args, const void *V, int64_t nseg, const ba_plan_info *info,

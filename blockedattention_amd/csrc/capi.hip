@@ -177,6 +177,7 @@ __attribute__((visibility("default"))) int ba_plan_wait(const void *mailbox, uin
     const auto t0 = std::chrono::steady_clock::now();
     for (uint64_t spins = 0;; ++spins) {
         if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == ticket) break;
+        __builtin_ia32_pause();                            // a polite spin: the sibling hardware thread gets the core
         if ((spins & 1023) == 1023 && timeout_us >= 0 &&
             std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count() > timeout_us)
             return BA_ERR_LAUNCH;
@@ -226,21 +227,6 @@ __attribute__((visibility("default"))) int ba_blocked_softmax_backward(void *pla
     if (H == 0 || Dsrc == 0 || nseg == 0) return BA_OK;
     if (!y || !dy || !dx) return BA_ERR_INVALID_ARG;
     return launch_softmax_backward(dtype, plan, nseg, y, dy, dx, H, Dsrc, scale, info, (hipStream_t)stream);
-}
-
-__attribute__((visibility("default"))) int ba_repack_operand(const void *src_plan, int src_which, int swap_dims,
-                                                             int column_major, const void *dst_plan, int dst_which,
-                                                             const ba_plan_info *dst_info, int64_t nseg, int dtype,
-                                                             const void *src, void *dst, int64_t H, int64_t Dsrc,
-                                                             int64_t Ddst, ba_stream_t stream) {
-    if (!src_plan || !dst_plan || nseg < 0 || nseg > (int64_t(1) << 30) || H < 0 || Dsrc < 0 || Ddst < 0)
-        return BA_ERR_INVALID_ARG;
-    if (src_which < 0 || src_which > 2 || dst_which < 0 || dst_which > 1) return BA_ERR_INVALID_ARG;
-    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
-    if (H == 0 || Ddst == 0 || nseg == 0) return BA_OK;
-    if (!dst || (Dsrc > 0 && !src)) return BA_ERR_INVALID_ARG;
-    return launch_repack(src_plan, src_which, swap_dims ? 1 : 0, column_major ? 1 : 0, dst_plan, dst_which, nseg, src, dst,
-                         H, Dsrc, Ddst, dst_info, (hipStream_t)stream);
 }
 
 __attribute__((visibility("default"))) int ba_gemm_softmax(void *plan, const ba_plan_info *info, int64_t nseg,

@@ -572,12 +572,13 @@ int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, c
     // pairs of 4 .. 16 row blocks, fused / product alone: Z = 16 1874 / 1307 us; two pairs taking turns 1795 / 1303;
     // Z = 3 (about three workgroups per compute unit) 1813 / 1201, but then ten pairs are in flight per die, B_g
     // leaves the die's L2 between a workgroup's passes and the launch reads 1.9 GB instead of 0.6.
-    // Hence: fused, one workgroup per row block and two pairs taking turns; the product alone, Z = 3 x 256 / pairs.
+    // Hence: fused, one workgroup per row block and two pairs taking turns; the product alone, about three workgroups
+    // per compute unit (Z = 3 x compute units / pairs).
     // BLOCKEDATTN_ROWBLOCK_Z and BLOCKEDATTN_ROWBLOCK_WEAVE override.
     static const int forced_z = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK_Z"); return e ? atoi(e) : 0; }();
     static const int forced_w = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK_WEAVE"); return e ? atoi(e) : 0; }();
     const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRbRows - 1) / kRbRows));
-    int64_t z = fused ? z_max : std::min<int64_t>(z_max, (3 * 256 + pairs - 1) / pairs);
+    int64_t z = fused ? z_max : std::min<int64_t>(z_max, (3 * (int64_t)device_cu_count() + pairs - 1) / pairs);
     if (forced_z > 0) z = std::min<int64_t>(z_max, forced_z);
     const int64_t weave = std::max<int64_t>(1, std::min<int64_t>(forced_w > 0 ? forced_w : (fused ? 2 : 1), pairs / kDies));
     pairs = (pairs / kDies + weave - 1) / weave * weave * kDies;       // whole turns

@@ -159,8 +159,11 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
                     }
                 }
             }
+            // every dimension and every area of a segment below 2^30: the kernels address a segment with 32-bit byte
+            // offsets (the products below cannot overflow: each factor is below 2^30 when they are formed)
             const int64_t lim = int64_t(1) << 30;
             bad = bad || m < 0 || n < 0 || k < 0 || m >= lim || n >= lim || k >= lim;
+            bad = bad || m * k >= lim || n * k >= lim || m * n >= lim;
             if (bad) { m = n = k = 0; }
         }
         const int32_t mi = (int32_t)m, ni = (int32_t)n, ki = (int32_t)k;

@@ -80,7 +80,7 @@ int64_t leading(const Tensor &t) {
 }
 
 struct Schedule;
-// Schedules derived from one schedule (padded / permuted shapes for the repacked GEMMs), made on first
+// Schedules derived from one schedule (permuted shapes for the two GEMMs of the backward pass), made on first
 // use and shared by every copy of the schedule, so that they live and die with its cache entry.
 struct Derived {
     std::mutex mu;

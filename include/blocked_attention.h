@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BA_ABI_VERSION 3
+#define BA_ABI_VERSION 4
 
 typedef void *ba_stream_t; /* hipStream_t */
 
@@ -208,29 +208,6 @@ int ba_gemm_softmax(void *plan, const ba_plan_info *info, int64_t nseg, int dtyp
                     ba_stream_t stream);
 
 /*
- * Repack of one 16-bit operand of every segment into the layout the MFMA
- * kernels read (rows of a multiple of 8 elements, zero padded), optionally
- * transposed.  The reference has no such step: it hands transposed layouts,
- * the two GEMMs of its backward pass (dA = dS B, dB = dS^T A,
- * csrc/sparseBlockedAttention.cpp:52-72) and any reduction length to one
- * generic kernel through transpose flags (csrc/cuda/spBlkGEMM.cu:424-817);
- * here the caller repacks into a scratch tensor of its own and runs
- * ba_varlen_gemm on the result.
- *
- * Destination: operand dst_which (0: the M x K operand, 1: the N x K operand)
- * of dst_plan, row-major at that plan's offsets, Ddst elements per head.
- * Source: operand src_which (0, 1, or 2: the M x N result) of src_plan, seen as
- * a matrix of that operand's dimensions, swapped if swap_dims, stored row-major
- * or, if column_major, column-major, at src_plan's offsets, Dsrc elements per
- * head.  destination[r][c] = source[r][c] where the source has that element,
- * 0 elsewhere.  Both plans must describe the same number of segments; dst_info
- * (optional) is the host summary of dst_plan.
- */
-int ba_repack_operand(const void *src_plan, int src_which, int swap_dims, int column_major, const void *dst_plan,
-                      int dst_which, const ba_plan_info *dst_info, int64_t nseg, int dtype, const void *src, void *dst,
-                      int64_t H, int64_t Dsrc, int64_t Ddst, ba_stream_t stream);
-
-/*
  * Varlen attention in one pass: out_g = softmax(scale * Q_g K_g^T) V_g per
  * segment and head, the M x N probabilities never written to memory.  It
  * stands in for the chain a caller of the reference runs for attention
@@ -262,6 +239,10 @@ int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg, int 
  * info == NULL, and give the same results.  Metadata the scheduler rejects
  * leaves `out` unwritten (there is no summary to report it through), so check
  * new metadata once with ba_plan_gemm + ba_plan_read.
+ * The FIRST call on a device looks up the buffer's address and sets kernel
+ * attributes (host-side calls that do not belong in a stream capture): make
+ * one call per device outside any capture, with any small batch, before the
+ * calls that are captured.
  * At most BA_STATIC_MAX_SEGMENTS segments: more returns BA_ERR_WORKSPACE.
  * All calls on one GPU share that GPU's buffer: calls that overlap on one GPU
  * (different streams or threads) race; calls on one stream do not.

@@ -61,7 +61,7 @@ def test_offsets_bit_exact_and_items_cover(dev, cfg):
     assert info["bad_segments"] == 0
 
 
-@pytest.mark.parametrize("cfg", [1, 3, 4, 5])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
 def test_lists_from_prefix_sums_are_exact(dev, cfg):
     w = workloads.make(cfg)
     a1, a2, ao = [dev_i64(a, dev) for a in oracle.lists_to_accum(w.M, w.N, w.K)]
@@ -74,8 +74,8 @@ def test_lists_from_prefix_sums_are_exact(dev, cfg):
 
 
 def test_lists_from_prefix_sums_large_and_degenerate(dev):
-    M = np.array([4097, 99991, 16777217, 3, 0, 1 << 20]); N = np.array([4095, 7, 3, 16777219, 0, 1 << 20])
-    K = np.array([127, 99989, 5, 2, 0, 1 << 20])
+    M = np.array([4097, 99991, 16777217, 3, 0, 1 << 15]); N = np.array([4095, 7, 3, 16777219, 0, 1 << 14])
+    K = np.array([127, 9989, 5, 2, 0, 1 << 14])
     a = [dev_i64(x, dev) for x in oracle.lists_to_accum(M, N, K)]
     m = torch.empty(6, dtype=torch.int64, device=dev); n = m.clone(); k = m.clone()
     info = capi.plan_gemm(6, dev, m, n, k, *a, mode=capi.META_FROM_ACCUM).read()
@@ -89,6 +89,21 @@ def test_lists_from_prefix_sums_large_and_degenerate(dev):
     om, on, ok, obad = oracle.accum_to_lists([0, 6, 12], [0, 10, 20], [0, 14, 29])
     assert info.bad_segments == obad == 1
     assert np.array_equal(m.cpu().numpy(), om) and np.array_equal(k.cpu().numpy(), ok)
+
+
+def test_segment_areas_of_2_to_the_30_elements_are_rejected(dev):
+    # every dimension is admissible, one area is not: the kernels address a segment with 32-bit byte offsets, so
+    # M K, N K and M N of a segment stay below 2^30 elements -- from lists and from prefix sums alike
+    for M, N, K in (([40000, 8], [40000, 8], [8, 8]), ([1 << 20, 8], [16, 8], [1 << 10, 8]), ([16, 8], [1 << 20, 8], [1 << 10, 8])):
+        plan = make_plan(dev, np.array(M), np.array(N), np.array(K), read=False)
+        assert plan.read(raise_on_bad=False).bad_segments == 1
+        a = [dev_i64(x, dev) for x in oracle.lists_to_accum(np.array(M), np.array(N), np.array(K))]
+        m = torch.empty(2, dtype=torch.int64, device=dev); n = m.clone(); k = m.clone()
+        plan = capi.plan_gemm(2, dev, m, n, k, *a, mode=capi.META_FROM_ACCUM)
+        assert plan.read(raise_on_bad=False).bad_segments == 1
+    # just below the limit is fine
+    plan = make_plan(dev, np.array([32767]), np.array([32768]), np.array([8]), read=False)
+    assert plan.read(raise_on_bad=False).bad_segments == 0
 
 
 def test_more_segments_than_one_scheduler_pass(dev):

@@ -149,7 +149,7 @@ def test_repeated_metadata_reuses_the_schedule(dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_autograd_16bit_through_the_repacked_gemms(dev, dtype):
+def test_autograd_16bit_through_the_any_layout_gemms(dev, dtype):
     # dA = dS B (reduction over N) and dB = dS^T A (over M) with N, M that are not multiples of 8
     import blockedAttention
     M, N, K = [5, 33, 16, 130], [7, 20, 64, 257], [8, 16, 24, 64]

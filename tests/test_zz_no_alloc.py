@@ -24,10 +24,18 @@ def both_ways(dev, M, N, K, H, dtype, scale, seed):
     want = torch.full((H, do), float("nan"), dtype=dtype, device=dev)
     capi.gemm_softmax(plan, Ad, Bd, want, H, d1, d2, do, scale)
     got = torch.full((H, do), float("nan"), dtype=dtype, device=dev)
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(dev)
+    # one call first: the code object is loaded and the buffer's address looked up (once per device); then two calls
+    # between which the DEVICE's free memory (hipMemGetInfo: whatever allocates, torch's allocator or the library
+    # itself) must not move
     capi.gemm_softmax_static(Md, Nd, Kd, Ad, Bd, got, H, d1, d2, do, scale)
     torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    before = torch.cuda.memory_allocated(dev)
+    got.fill_(float("nan"))
+    capi.gemm_softmax_static(Md, Nd, Kd, Ad, Bd, got, H, d1, d2, do, scale)
+    capi.gemm_softmax_static(Md, Nd, Kd, Ad, Bd, got, H, d1, d2, do, scale)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before, "the device's free memory moved across the calls"
     assert torch.cuda.memory_allocated(dev) == before
     assert torch.equal(got.view(torch.int16), want.view(torch.int16)), "static plan and caller's plan disagree"
     assert_probs_close(got, oracle.per_segment_torch(A, B, M, N, K, scale), "static")
