@@ -21,7 +21,8 @@ region, and `traffic` from the tracked rocprofv3 summary of the same kernel and
 workload under profiles/ (null when there is none).
 `cpu_baseline` is the per-segment torch matmul + softmax path on the host cores.
 `others` carries the same GPU figures for the remaining configurations, each
-with its own hbm_frac (at least 100 timed iterations after 20 warm-up ones).
+with its own hbm_frac (at least 100 timed iterations after 20 warm-up ones);
+configurations 3 and 4 also at seeds 1 and 2 (`seeds`: other segment sizes).
 """
 import argparse
 import json
@@ -74,13 +75,13 @@ def parse():
 class Case:
     """One configuration resident on the GPU, with its plan."""
 
-    def __init__(self, cfg, dev):
+    def __init__(self, cfg, dev, seed=0):
         import torch
         from blockedattention_amd import capi, workloads
         self.torch, self.capi = torch, capi
-        self.w = w = workloads.make(cfg)
+        self.w = w = workloads.make(cfg, seed)
         self.cfg = cfg
-        A, B = w.operands()
+        A, B = w.operands(seed)
         self.A_host, self.B_host = A, B
         self.A, self.B = A.to(dev), B.to(dev)
         i64 = lambda a: torch.from_numpy(a).to(dev)
@@ -438,6 +439,18 @@ def main():
             others[f"cfg{cfg}"] = f
             del c
             torch.cuda.empty_cache()
+            if cfg in (3, 4):
+                # the same configuration drawn from two more seeds: other segment sizes, other values
+                f["seeds"] = {}
+                for seed in (1, 2):
+                    c = Case(cfg, dev, seed)
+                    c.check()
+                    k_us = c.event_us(c.fused, steps, warm)
+                    f["seeds"][str(seed)] = {
+                        "kernel_us": round(k_us, 3), "call_us": round(c.wall_us(c.step, steps, warm), 3),
+                        "pair_bytes": c.w.pair_bytes(), "hbm_frac": round(c.w.pair_bytes() / k_us * 1e-3 / HBM_PEAK_GBS, 4)}
+                    del c
+                    torch.cuda.empty_cache()
         line["others"] = others
     print(json.dumps(line))
     return 0
