@@ -21,7 +21,13 @@ region, and `traffic` from the tracked rocprofv3 summary of the same kernel and
 workload under profiles/ (null when there is none).
 `cpu_baseline` is the per-segment torch matmul + softmax path on the host cores.
 `others` carries the same GPU figures for the remaining configurations, each
-with its own hbm_frac (at least 100 timed iterations after 20 warm-up ones);
+with its own hbm_frac (at least 100 timed iterations after 20 warm-up ones).
+There `call_us` is one call on fresh metadata, host clock: for a small batch (at
+most 512 segments, 1024 (segment, head) pairs, 2^24 results) the single launch of
+ba_gemm_softmax_static (`call_is_single_launch`), else ba_plan_gemm +
+ba_gemm_softmax; `plan_call_us` is the latter pair whatever the size,
+`one_call_entry_us` the former entry whatever the size, `kernel_us` the
+plan-driven fused kernel alone;
 configurations 3 and 4 also at seeds 1 and 2 (`seeds`: other segment sizes).
 """
 import argparse
@@ -122,7 +128,17 @@ class Case:
                           *dims, i32(1), i32(1), st)
         self._a_soft = (p.ptr, p._hint(), i64(w.nseg), code, c._ptr(self.scores), c._ptr(self.out), i64(w.heads),
                         i64(w.Dout), f32(w.scale), st)
+        # the one-call entry: metadata and operands in, probabilities and prefix sums out (its plan, where it
+        # needs one, lives in the library)
+        self._a_static = (i64(w.nseg), i32(c.META_FROM_LISTS), c._ptr(self.M), c._ptr(self.N), c._ptr(self.K),
+                          c._ptr(self.acc[0]), c._ptr(self.acc[1]), c._ptr(self.acc[2]), code, c._ptr(self.A), c._ptr(self.B),
+                          c._ptr(self.out), code, *dims, f32(w.scale), st)
+        # batches the library runs as ONE launch through that entry (no scheduler launch, no plan)
+        # (the library's rule: at most 512 segments, 1024 pairs, 2^24 results and 2^24 operand values)
+        self.single_launch = (w.nseg <= 512 and w.nseg * w.heads <= 1024 and w.heads * w.Dout <= 1 << 24 and
+                              w.heads * (w.Dm1 + w.Dm2) <= 1 << 24)
         for st_code, what in ((lib.ba_plan_gemm(*self._a_sched), "ba_plan_gemm"),
+                              (lib.ba_gemm_softmax_static(*self._a_static), "ba_gemm_softmax_static"),
                               (lib.ba_gemm_softmax(*self._a_fused), "ba_gemm_softmax"),
                               (lib.ba_varlen_gemm(*self._a_gemm), "ba_varlen_gemm"),
                               (lib.ba_blocked_softmax(*self._a_soft), "ba_blocked_softmax"),
@@ -147,9 +163,21 @@ class Case:
     def attention(self):
         self._lib.ba_varlen_attention(*self._a_att)
 
-    def step(self):
+    def plan_step(self):
         self._lib.ba_plan_gemm(*self._a_sched)
         self._lib.ba_gemm_softmax(*self._a_fused)
+
+    def one_call(self):
+        self._lib.ba_gemm_softmax_static(*self._a_static)
+
+    def step(self):
+        """One call on fresh metadata: the single launch where the batch is small enough for it, else scheduler +
+        fused kernel through the plan."""
+        if self.single_launch:
+            self._lib.ba_gemm_softmax_static(*self._a_static)
+        else:
+            self._lib.ba_plan_gemm(*self._a_sched)
+            self._lib.ba_gemm_softmax(*self._a_fused)
 
     def unfused(self):
         self._lib.ba_varlen_gemm(*self._a_gemm)
@@ -241,8 +269,9 @@ class Case:
 
     def timed_region(self, steps, warmup):
         """The contract's timed region: `warmup` untimed steps, then exactly `steps` steps between two
-        synchronisations.  A step = scheduler + fused kernel; HIP events on the launch stream bracket the fused
-        kernel of every step.  Returns (wall us per step, mean fused-kernel us)."""
+        synchronisations.  A step = scheduler + fused kernel (one launch doing both for a small batch); HIP events
+        on the launch stream bracket the fused kernel of every step.  Returns (wall us per step, mean fused-kernel
+        us)."""
         torch = self.torch
         for _ in range(warmup):
             self.step()
@@ -250,9 +279,13 @@ class Case:
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for e0, e1 in ev:
-            self._lib.ba_plan_gemm(*self._a_sched)
-            e0.record()
-            self._lib.ba_gemm_softmax(*self._a_fused)
+            if self.single_launch:
+                e0.record()
+                self._lib.ba_gemm_softmax_static(*self._a_static)
+            else:
+                self._lib.ba_plan_gemm(*self._a_sched)
+                e0.record()
+                self._lib.ba_gemm_softmax(*self._a_fused)
             e1.record()
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e6 / steps
@@ -266,6 +299,9 @@ class Case:
             "workload": w.name, "dtype": str(w.dtype).replace("torch.", ""),
             "kernel_us": round(k_us, 3),
             "call_us": round(self.wall_us(self.step, steps, warmup), 3),
+            "call_is_single_launch": self.single_launch,
+            "plan_call_us": round(self.wall_us(self.plan_step, steps, warmup), 3),
+            "one_call_entry_us": round(self.wall_us(self.one_call, steps, warmup), 3),
             "scheduler_us": round(self.event_us(self.schedule, steps, warmup), 3),
             "pair_bytes": w.pair_bytes(), "flops": w.flops,
             "GBps": round(w.pair_bytes() / k_us * 1e-3, 1), "TFLOPs": round(w.flops / k_us * 1e-6, 2),

@@ -23,7 +23,7 @@ OBJDIR = os.path.join(PKG, "lib", "obj")
 LIB_PATH = os.path.join(LIBDIR, "libblockedattn_hip.so")
 EXT_PATH = os.path.join(PKG, "blockAttention" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
-HIP_SOURCES = ["scheduler.hip", "gemm_softmax.hip", "tile_kernel.hip", "rowblock_kernel.hip", "rowpipe_kernel.hip", "softmax.hip", "gemm_generic.hip", "gemm_any16.hip", "attention.hip", "capi.hip"]
+HIP_SOURCES = ["scheduler.hip", "gemm_softmax.hip", "onecall_kernel.hip", "tile_kernel.hip", "rowblock_kernel.hip", "rowpipe_kernel.hip", "softmax.hip", "gemm_generic.hip", "gemm_any16.hip", "attention.hip", "capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

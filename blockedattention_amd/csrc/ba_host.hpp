@@ -60,6 +60,19 @@ int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, c
 // row blocks sharing one stream of B_g.  Same conditions as launch_rowblocks.
 int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_info *info, hipStream_t stream);
 // fp16 / bf16 in any layout and alignment (gemm_any16.hip: both operands staged through LDS, MFMA)
+// Fused GEMM + softmax of a batch of at most kOneCallMaxSegments segments in one launch that reads the metadata
+// itself (mode 0: sizes given, prefix sums written; mode 2: both given); no plan.  Every workgroup redoes the
+// scheduler's sums and runs with the widest build's registers and LDS window, so it only pays while the batch has
+// few (segment, head) pairs: measured against scheduler + plan-driven kernels, 64 segments x 1 head 4.5 against
+// 8.3 us, 256 x 2 heads 9.2 against 12.9, 256 x 4 equal (16.5 / 16.2), 256 x 8 30.5 against 21.0.
+constexpr int kOneCallMaxSegments = 512;
+constexpr int kOneCallMaxPairs = 1024;
+// ... and while the call is short enough for a launch to matter: with more than 2^24 results or operand values
+// (32 MiB of 16-bit data, at least some 10 us of kernel) the plan-driven kernels' better fit to the batch (work
+// order, row-block kernels for large segments, the lean build) is worth more than the launch saved.
+constexpr int64_t kOneCallMaxElements = int64_t(1) << 24;
+int launch_onecall(int dtype, const RunArgs &args, int mode, const int64_t *M, const int64_t *N, const int64_t *K,
+                   int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream);
 int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 // fp32, fp64 and the integer types (gemm_generic.hip); dtype: ba_dtype
 int launch_gemm_generic(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);

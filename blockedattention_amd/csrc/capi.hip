@@ -1,6 +1,7 @@
 // extern "C" entry points of libblockedattn_hip.so: argument checks, flag
 // derivation and kernel launches.  No allocation, no host synchronisation
 // except ba_plan_read.
+#include <stdlib.h>
 #include <string.h>
 
 #include <chrono>
@@ -255,6 +256,18 @@ __attribute__((visibility("default"))) int ba_gemm_softmax_static(int64_t nseg, 
     if (nseg > BA_STATIC_MAX_SEGMENTS) return BA_ERR_WORKSPACE;
     if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
     if (out_dtype != dtype && out_dtype != BA_F32) return BA_ERR_UNSUPPORTED;
+    // Small batches: one launch that reads the metadata itself; neither the scheduler nor the plan buffer is used.
+    static const bool onecall = [] { const char *e = getenv("BLOCKEDATTN_ONECALL"); return !e || atoi(e) != 0; }();
+    if (onecall && nseg >= 1 && nseg <= kOneCallMaxSegments && nseg * H <= kOneCallMaxPairs && mode != BA_META_FROM_ACCUM &&
+        H > 0 && Dout > 0 && H * Dout <= kOneCallMaxElements && H * (Dm1 + Dm2) <= kOneCallMaxElements) {
+        if (mode < 0 || mode > 2 || !MList || !NList || !KList) return BA_ERR_INVALID_ARG;
+        if (mode == BA_META_GIVEN && (!accum1 || !accum2 || !accumOut)) return BA_ERR_INVALID_ARG;
+        if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
+        RunArgs args{nullptr, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, 0, (int)nseg};
+        args.flags |= mfma_flag(args);
+        if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
+        return launch_onecall(dtype, args, mode, MList, NList, KList, accum1, accum2, accumOut, (hipStream_t)stream);
+    }
     void *plan = static_plan_buffer();
     if (!plan) return BA_ERR_LAUNCH;
     // The scheduler rewrites the whole header (run-error counter included), every record and every list entry

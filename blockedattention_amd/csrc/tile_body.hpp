@@ -75,35 +75,10 @@ template <int N> __device__ __forceinline__ void wait_vm() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// One workgroup of the tile kernel: `block` is its index among the kernel's workgroups (it decides die,
-// pair and row block), lds its kStages * kTileChunkBytes bytes of LDS (1 KiB aligned).
+// The row blocks z0, z0 + zdim, ... (128 rows each) of one segment and head, by one workgroup of kTileThreads
+// work-items; lds = its kStages * kTileChunkBytes bytes of LDS (1 KiB aligned).
 template <int DT, bool FUSED, bool F32OUT>
-__device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned block, unsigned char *lds) {
-    const int die = block % kDies, slot = block / kDies;
-    const int pair = (slot / zdim) * kDies + die;
-    const int z0 = slot % zdim;
-    const int H = (int)a.H;
-    const PlanRO pv = plan_ro(a.plan, a.nseg);
-    const bool ok = header_ok(a);
-    if (!ok) {
-        if (!(a.flags & kFlagQuiet) && block == 0 && threadIdx.x == 0)
-            atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
-        return;
-    }
-    // pairs = (entries of the work list, padded to a multiple of the die count) x heads, entry fastest,
-    // and the entries rotated by the head: die d works on entries = (d + h) mod 8 of head h, so over the
-    // heads every die sees every segment about equally often, however unequal the segments are.
-    const int entries = a.list < 0 ? a.nseg : (int)((ConstHdr)(uintptr_t)a.plan)->totals[a.list];
-    const int padded = (entries + kDies - 1) / kDies * kDies;
-    if (entries <= 0 || pair >= padded * H) return;
-    const int h = pair / padded;
-    const int entry = (pair % padded + h) % padded;
-    if (entry >= entries) return;
-    bool valid;
-    const Seg s = load_listed(pv, entry, h, a, valid);
-    if (!valid) return;
-    const int kind = s.kind;
-    if (!tile_segment(kind, s.N, s.K)) return;
+__device__ __forceinline__ void tile_rows(const RunArgs &a, const Seg &s, int z0, int zdim, unsigned char *lds) {
     const int M = s.M, N = s.N, K = s.K;
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
     const int wave = uniform((int)(threadIdx.x >> 6));
@@ -117,8 +92,10 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
     constexpr int kStoreInsts = (F32OUT ? 2 : 1) * kRT * 4;  // per store iteration and wavefront
     const u32x4 zero = {0u, 0u, 0u, 0u};
 
-    const int nslab = (K + kSlabK - 1) / kSlabK;
-    const int nspan = (K + kSpanK - 1) / kSpanK;
+    // K = 0: one slab of zeros (no fill is issued for it, the stages are cleared instead), so that the sweeps
+    // run and the rows come out as zeros, or as 1/N from the fused call
+    const int nslab = K > 0 ? (K + kSlabK - 1) / kSlabK : 1;
+    const int nspan = K > 0 ? (K + kSpanK - 1) / kSpanK : 1;
     const int ncb = (N + kTileCols - 1) / kTileCols;
     const int per_sweep = ncb * nslab;
     const int total = (FUSED ? 2 : 1) * per_sweep;
@@ -152,6 +129,11 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
         }
     };
 
+    if (K == 0) {
+        for (int i = threadIdx.x; i < kStages * kTileChunkBytes / 16; i += kTileThreads)
+            reinterpret_cast<u32x4 *>(lds)[i] = zero;
+        __syncthreads();
+    }
     for (int rb = z0; rb * kTileRows < M; rb += zdim) {
         const int row0 = rb * kTileRows + wave * kTileWaveRows;     // first row of this wavefront
         const bool active = row0 < M;
@@ -168,6 +150,8 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
                         if (k0 + ks * 32 + rg * 8 >= K) v = zero;        // ragged last k-step
                         if (negate) v ^= u32x4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
                         af[rt][ks] = v;
+                    } else if (K == 0 && ks == 0) {
+                        af[rt][0] = zero;                                // the one k-step of a K = 0 segment
                     }
                 }
             }
@@ -371,5 +355,37 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
     }
 }
 
+
+// One workgroup of the tile kernel: `block` is its index among the kernel's workgroups (it decides die,
+// pair and row block), lds its kStages * kTileChunkBytes bytes of LDS (1 KiB aligned).
+template <int DT, bool FUSED, bool F32OUT>
+__device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned block, unsigned char *lds) {
+    const int die = block % kDies, slot = block / kDies;
+    const int pair = (slot / zdim) * kDies + die;
+    const int z0 = slot % zdim;
+    const int H = (int)a.H;
+    const PlanRO pv = plan_ro(a.plan, a.nseg);
+    const bool ok = header_ok(a);
+    if (!ok) {
+        if (!(a.flags & kFlagQuiet) && block == 0 && threadIdx.x == 0)
+            atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+        return;
+    }
+    // pairs = (entries of the work list, padded to a multiple of the die count) x heads, entry fastest,
+    // and the entries rotated by the head: die d works on entries = (d + h) mod 8 of head h, so over the
+    // heads every die sees every segment about equally often, however unequal the segments are.
+    const int entries = a.list < 0 ? a.nseg : (int)((ConstHdr)(uintptr_t)a.plan)->totals[a.list];
+    const int padded = (entries + kDies - 1) / kDies * kDies;
+    if (entries <= 0 || pair >= padded * H) return;
+    const int h = pair / padded;
+    const int entry = (pair % padded + h) % padded;
+    if (entry >= entries) return;
+    bool valid;
+    const Seg s = load_listed(pv, entry, h, a, valid);
+    if (!valid) return;
+    const int kind = s.kind;
+    if (!tile_segment(kind, s.N, s.K)) return;
+    tile_rows<DT, FUSED, F32OUT>(a, s, z0, zdim, lds);
+}
 
 }  // namespace ba

@@ -126,3 +126,10 @@ def test_nearly_empty_last_row_block_under_load(dev):
     M = np.array([267, 523, 11, 290]); N = np.array([1483, 2571, 900, 2594]); K = np.array([128, 128, 64, 128])
     for rep in range(2):
         run_all(dev, M, N, K, 16, torch.float16, 0.05, seed=21 + rep)
+
+
+def test_k_zero_in_the_tile_kernel(dev):
+    # without the host summary, and next to a K = 136 segment, the large segments run in the tile kernel: K = 0
+    # has no operand bytes there either, and the rows are zeros (product) or 1/N (fused pair)
+    run_all(dev, [40, 200, 70], [300, 130, 260], [0, 0, 64], 2, torch.float16, 0.2, summary=False)
+    run_all(dev, [40, 200, 70], [300, 130, 260], [0, 0, 136], 2, torch.bfloat16, 0.2)
