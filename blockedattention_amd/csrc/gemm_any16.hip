@@ -4,15 +4,25 @@
 // alignment.  The backward of the product is two such calls (csrc/sparseBlockedAttention.cpp:52-72: dA = dS B
 // reduces over N, dB = dS^T A over M, with dS and the saved operands read as they lie).
 //
-// Workgroup = 64 rows x 64 columns of one segment and head at a time, k in chunks of 64.  Both operand chunks go
-// through LDS with a row pitch of 160 bytes.  Staging reads 16 bytes per lane along whatever dimension is contiguous
+// Workgroup = 128 rows x 128 columns of one segment and head at a time (64 x 64 in the build for batches of short
+// segments), k in chunks of 64.  Both operand chunks go through LDS with a row pitch of 160 bytes (288 for 128 rows
+// stored k-major).  Staging reads 16 bytes per lane along whatever dimension is contiguous
 // in memory, at any 2-byte alignment, through a buffer descriptor that spans exactly the segment (rows past its
 // end read as zeros), and writes them to LDS as they come: an operand that is not transposed lies there as
 // [row][k] and is read 16 bytes per lane; an operand stored k-major lies there k-major and the matrix operand is
 // gathered by the transposing LDS read (ds_read_b64_tr_b16, four k of one row per lane).  Each wavefront
-// then computes 16 rows x 64 columns as four 16 x 16 tiles with v_mfma_f32_16x16x32 (fp32 sums).  Column slot n of
-// tile t is column 4 n + t, so a lane owns four consecutive columns of each of its rows and the sixteen lanes of a
-// row group write 128 contiguous bytes.
+// then computes 16 or 32 rows x 64 or 128 columns as 16 x 16 tiles with v_mfma_f32_16x16x32 (fp32 sums).  Column slot n of
+// tile t is column 4 n + t (8 n + t in the 128-column step), so a lane owns four (eight) consecutive columns of
+// each of its rows and the sixteen lanes of a row group write 128 (256) contiguous bytes.
+//
+// What bounds it, measured on 16 segments x 16 heads of 1024..4096 rows and columns, K = 128, both operands k-major
+// (rocprofv3 counters): the first pipelined build moved 4.7 GB in and 4.6 GB out of memory for 0.34 GB of operands
+// and 3.86 GB of results and spent 56 % of its wave cycles in s_waitcnt.  Keeping the X chunks of a round in LDS
+// (K <= 128) took the reads to 1.0 GB and the kernel from 1930 to 1660 us; the writes stay at 1.18 x the result
+// (rows start at any 2-byte phase, so every 256-byte piece ends in partial lines), which is what separates it from
+// the plain-layout kernel (1210 us) that writes whole lines through an LDS ring.
+#include <stdlib.h>
+
 #include <algorithm>
 
 #include "ba_gemm_common.hpp"
@@ -20,7 +30,6 @@
 namespace ba {
 
 constexpr int kAnyThreads = 256;
-constexpr int kAnyWaves = kAnyThreads / 64;
 constexpr int kAnyTile = 64;                         // rows and columns per workgroup step, k per chunk
 constexpr int kAnyPitch = (kAnyTile + 16) * 2;       // bytes per LDS row: 160 = 16 * (2 * odd), the pitch at which the
 // 16-byte operand reads (served 32 lanes, 512 bytes at a time) and the transposing 8-byte reads meet no bank conflict
@@ -28,6 +37,8 @@ constexpr int kAnyPitch = (kAnyTile + 16) * 2;       // bytes per LDS row: 160 =
 // Sixteen consecutive elements of the segment from byte offset `off` on (kNoLine: zeros).  Two 16-byte loads where
 // they lie inside the segment; a piece that reaches past its end is fetched element by element, the hardware
 // returning zero for those outside (a wide load that crosses the end of the descriptor's range is dropped whole).
+constexpr int kDies = 8;
+constexpr int kAnyDieBlock = 16;
 constexpr uint32_t kNoLine = 0x80000000u;
 union Line16 {
     u32x4 v[2];
@@ -47,71 +58,107 @@ __device__ __forceinline__ Line16 load_line16(__amdgpu_buffer_rsrc_t res, uint32
     return x;
 }
 
-// One 64 x 64 chunk of an operand on its way into LDS as dst[row][k], in two steps so that the loads of the next
-// chunk can be in flight while the matrix instructions work on the current one.  The operand is `rows` x K (or,
-// transposed, stored K x rows); the chunk starts at row r0, reduction index k0.  Thread t takes sixteen
-// consecutive elements along the contiguous dimension of line t / 4.
+// One chunk of an operand (R rows x 64 k, R = 16 * PARTS) on its way into LDS, in two steps so that the loads of
+// later chunks can be in flight while the matrix instructions work on the current one.  The operand is `rows` x K
+// (or, transposed, stored K x rows); the chunk starts at row r0, reduction index k0.  A chunk is 4 R slots of
+// sixteen consecutive elements along the contiguous dimension: not transposed, slot s is k part s % 4 of row s / 4;
+// transposed, row part s % PARTS of k line s / PARTS.  A thread takes the slots tid, tid + 256, ...
+template <int PARTS>
 __device__ __forceinline__ Line16 fetch_chunk16(__amdgpu_buffer_rsrc_t res, bool transposed, int rows, int K, int r0, int k0,
-                                                int tid) {
-    const int line = tid >> 2, part = (tid & 3) * 16;
+                                                int slot) {
+    const int line = transposed ? slot / PARTS : slot >> 2, part = (transposed ? slot % PARTS : slot & 3) * 16;
     const uint32_t bytes = (uint32_t)(rows * K) * 2u;
-    // not transposed: line = row, the sixteen elements run along k; transposed: line = k, they run along the rows
     const int row = r0 + (transposed ? part : line), k = k0 + (transposed ? line : part);
     const int lead = transposed ? k * rows + row : row * K + k;
     return load_line16(res, row < rows && k < K ? (uint32_t)lead * 2u : kNoLine, bytes);
 }
-// Into LDS.  An operand that is not transposed lies as dst[row][k].  A transposed one stays k-major, dst[k][..], and
-// the matrix operand is gathered by transposing reads (lds_tr8 below): 16-byte writes here instead of sixteen 2-byte
-// ones.  X (rows of the output) keeps its rows in order.  Y (columns of the output) permutes each group of sixteen
-// columns, 16 a + 4 b + t -> position 16 t + 4 a + b, so that the lane that reads position 16 t + i of a row gets
-// column 4 i + t: the columns a lane stores side by side (see the kernel).
-template <bool PERMUTE>
+// Into LDS.  An operand that is not transposed lies as dst[row][k] (pitch kAnyPitch).  A transposed one stays
+// k-major, dst[k][..] (pitch PITCH_T), and the matrix operand is gathered by transposing reads (lds_tr8 below):
+// 16-byte writes here instead of sixteen 2-byte ones.  X (rows of the output) keeps its rows in order.  Y (columns
+// of the output) permutes its columns so that the lane that reads position 16 t + i of a k line (slot i of tile t)
+// gets the columns a lane stores side by side: column 4 i + t of a 64-column step (16 a + 4 b + t -> position
+// 16 t + 4 a + b), column 8 i + t of a 128-column step.
+template <bool PERMUTE, int PARTS, int PITCH_T>
 __device__ __forceinline__ void put_chunk16(Line16 x, bool transposed, int rows, int K, int r0, int k0, unsigned char *dst,
-                                            int tid) {
-    const int line = tid >> 2, part = (tid & 3) * 16;
+                                            int slot) {
+    const int line = transposed ? slot / PARTS : slot >> 2, part = (transposed ? slot % PARTS : slot & 3) * 16;
     const int valid = transposed ? rows - (r0 + part) : K - (k0 + part);   // elements of the line from here on
+    if (valid < 16) {                                 // only the chunk at the end of the rows or of K
 #pragma unroll
-    for (int i = 0; i < 16; ++i) x.e[i] = i < valid ? x.e[i] : (uint16_t)0;
-    if (!PERMUTE || !transposed) {
+        for (int i = 0; i < 16; ++i) x.e[i] = i < valid ? x.e[i] : (uint16_t)0;
+    }
+    if (!transposed) {
         u32x4 *d = reinterpret_cast<u32x4 *>(dst + line * kAnyPitch + part * 2);
         d[0] = x.v[0];
         d[1] = x.v[1];
+    } else if (!PERMUTE) {
+        u32x4 *d = reinterpret_cast<u32x4 *>(dst + line * PITCH_T + part * 2);
+        d[0] = x.v[0];
+        d[1] = x.v[1];
+    } else if (PARTS == 8) {
+        // 128 columns: column 8 i + t -> position 16 t + i (eight tiles; a lane stores eight columns side by side)
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(&x);
+        unsigned char *d = dst + line * PITCH_T + (part >> 4) * 4;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {                 // elements t and 8 + t of the thread's sixteen
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+            *reinterpret_cast<uint32_t *>(d + 32 * t) = __builtin_amdgcn_perm(w[4 + (t >> 1)], w[t >> 1], sel);
+        }
     } else {
         const uint32_t *w = reinterpret_cast<const uint32_t *>(&x);
+        unsigned char *d = dst + line * PITCH_T + ((part >> 4) & 3) * 8;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {                 // elements t, 4 + t, 8 + t, 12 + t of the thread's sixteen
             const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
             const uint32_t lo = __builtin_amdgcn_perm(w[2 + (t >> 1)], w[t >> 1], sel);
             const uint32_t hi = __builtin_amdgcn_perm(w[6 + (t >> 1)], w[4 + (t >> 1)], sel);
-            *reinterpret_cast<u32x2 *>(dst + line * kAnyPitch + 32 * t + (part >> 2) * 2) = u32x2{lo, hi};
+            *reinterpret_cast<u32x2 *>(d + 32 * t) = u32x2{lo, hi};
         }
     }
 }
 // Eight k of one row (column) of a k-major chunk as matrix operand: two transposing reads of four k each.  In a
 // group of sixteen lanes, lane 4 e + a points at positions 4 a .. 4 a + 3 of k row e, and lane i receives position
 // i of the four k rows; p is this lane's address for the first four k, the next four lie four rows on.
+template <int PITCH_T>
 __device__ __forceinline__ u32x4 lds_tr8(const unsigned char *p) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 *LdsPtr;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(uintptr_t)p);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(uintptr_t)(p + 4 * kAnyPitch));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(uintptr_t)(p + 4 * PITCH_T));
     const u32x2 l = __builtin_bit_cast(u32x2, lo), h = __builtin_bit_cast(u32x2, hi);
     return u32x4{l[0], l[1], h[0], h[1]};
 }
 
-template <int DT>
-__global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
-    __shared__ __attribute__((aligned(16))) unsigned char sX[kAnyTile * kAnyPitch];
-    __shared__ __attribute__((aligned(16))) unsigned char sY[kAnyTile * kAnyPitch];
+// Workgroup barrier that waits for this wavefront's LDS traffic only: __syncthreads() would also wait for every
+// global load in flight, i.e. for the chunks that were just requested for the NEXT steps.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// LDS bytes of one operand buffer holding R = 64 or 128 rows x 64 k in either layout
+template <int R> struct AnyBuf {
+    static constexpr int pitch_t = (R + 16) * 2;          // k-major: 160 or 288 bytes = 16 * (2 * odd)
+    static constexpr int bytes = R * kAnyPitch > kAnyTile * pitch_t ? R * kAnyPitch : kAnyTile * pitch_t;
+};
+
+// RT = 16-row tiles per wavefront (the workgroup's step covers 64 RT rows), CG = groups of 64 columns per step.
+// The loads of a step are issued two steps ahead into registers, the chunks alternate between two LDS buffers:
+// one barrier per step, and two steps' worth of loads in flight per workgroup while it computes.  The kernel is
+// bound by operand traffic out of L2 (a 64 x 64 step fetches 16 KiB for 32 matrix instructions), which the
+// 128 x 128 step halves per result.
+template <int DT, int RT, int CG, bool T1, bool T2>
+__global__ __launch_bounds__(kAnyThreads, RT * CG >= 4 ? 2 : 4) void gemm_any16_kernel(RunArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char any_lds[];
+    constexpr int kRows = kAnyTile * RT, kCols = kAnyTile * CG;
+    constexpr int kPitchXT = AnyBuf<kRows>::pitch_t, kPitchYT = AnyBuf<kCols>::pitch_t;
+    constexpr int kBufBytes = AnyBuf<kRows>::bytes + AnyBuf<kCols>::bytes;
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
     const int nseg = hdr->nseg;
-    const int64_t per_head = hdr->att_blocks64;       // 64-row rounds per head (= the row-block prefix's last entry)
+    const int64_t per_head = RT == 2 ? hdr->att_blocks128 : hdr->att_blocks64;   // row rounds per head
     if (!header_ok(a)) {
         report_mismatch(a);
         return;
     }
     // Two grids.  With the batch's totals on the host (ride_slots = 1): one workgroup per existing
-    // (segment, 64-row round, head), head fastest, found by a search in the plan's row-block prefix.  Without:
+    // (segment, row round, head), head fastest, found by a search in the plan's row-block prefix.  Without:
     // (head, segment, z) or (segment, head, z), workgroup z taking the rounds z, z + gridDim.z, ...
     const bool head_fast = a.flags & kFlagHeadFast;
     // (a step past any segment's round count, small enough that first_round + step cannot overflow)
@@ -119,11 +166,17 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
     int g, first_round, round_step;
     int64_t h;
     if (a.ride_slots) {
-        const int32_t *pfx = plan_rowblocks(a.plan, nseg, 0);
+        const int32_t *pfx = plan_rowblocks(a.plan, nseg, RT == 2 ? 1 : 0);
+        // Workgroups go to the eight dies round-robin by their index, and each die has its own L2.  The work items
+        // (head slowest, then segment, then row round) are dealt to the dies in blocks of kAnyDieBlock consecutive
+        // items: the workgroups a die runs together are then neighbouring row rounds of one segment and head, which
+        // read the same Y, so Y comes out of that die's L2 instead of being streamed from memory once per round.
         const int64_t u = blockIdx.x;
-        if (u >= per_head * a.H) return;
-        h = u % a.H;                                   // consecutive workgroups: the heads of one round, one shape
-        const int item = (int)(u / a.H);
+        const int64_t slot = u / kDies;
+        const int64_t v = ((slot / kAnyDieBlock) * kDies + u % kDies) * kAnyDieBlock + slot % kAnyDieBlock;
+        if (v >= per_head * a.H) return;
+        h = v / per_head;
+        const int item = (int)(v % per_head);
         g = prefix_search(pfx, nseg, item);
         first_round = item - ((ConstI32)(uintptr_t)pfx)[g];
         round_step = rounds_never_again;
@@ -141,84 +194,177 @@ __global__ __launch_bounds__(kAnyThreads) void gemm_any16_kernel(RunArgs a) {
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = lane_id(), n = lane & 15, q = lane >> 4;
-    const bool t1 = a.flags & kFlagTranspose1, t2 = a.flags & kFlagTranspose2;
+    constexpr bool t1 = T1, t2 = T2;                  // the layouts are part of the build: no branch on them in the loop
     const __amdgpu_buffer_rsrc_t resX = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(reinterpret_cast<const uint16_t *>(a.A) + h * a.Dm1 + rec.off1), 0, M * K * 2, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t resY = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(reinterpret_cast<const uint16_t *>(a.B) + h * a.Dm2 + rec.off2), 0, N * K * 2, kRsrcFlags);
     uint16_t *os = reinterpret_cast<uint16_t *>(a.out) + h * a.Dout + rec.offO;
     const int nkc = (K + kAnyTile - 1) / kAnyTile;
-    // operand addresses of this lane inside a chunk: A operand = row 16 wave + n of X, B operand of tile t =
-    // row 4 n + t of Y (column slot n of tile t is column 4 n + t), eight k from 8 q on
-    const unsigned char *xa = sX + (16 * wave + n) * kAnyPitch + q * 16;
-    const unsigned char *ya = sY + (4 * n) * kAnyPitch + q * 16;
+    // operand offsets of this lane inside a buffer: A operand of row tile rt = row 16 (RT wave + rt) + n of X,
+    // B operand of tile t = row 4 n + t of Y (64-column step; 8 n + t in the 128-column step: column slot n of tile t
+    // is that column), eight k from 8 q on
+    const int xa = (16 * RT * wave + n) * kAnyPitch + q * 16;
+    const int ya = AnyBuf<kRows>::bytes + ((CG == 2 ? 8 : 4) * n) * kAnyPitch + q * 16;
     // the same from k-major chunks (transposed operands): k row 8 q + n / 4 of the step, positions 4 (n % 4) .. of the
-    // wavefront's sixteen rows (X) or of tile t's sixteen positions (Y, + 32 t bytes)
-    const unsigned char *xt = sX + (8 * q + (n >> 2)) * kAnyPitch + (16 * wave + 4 * (n & 3)) * 2;
-    const unsigned char *yt = sY + (8 * q + (n >> 2)) * kAnyPitch + (4 * (n & 3)) * 2;
+    // row tile's sixteen rows (X) or of tile t's sixteen positions (Y, + 32 t bytes)
+    const int xt = (8 * q + (n >> 2)) * kPitchXT + (16 * RT * wave + 4 * (n & 3)) * 2;
+    const int yt = AnyBuf<kRows>::bytes + (8 * q + (n >> 2)) * kPitchYT + (4 * (n & 3)) * 2;
 
-    // lane (n, q): rows 16 wave + 4 q + i, columns 64 cb + 4 n .. + 3; clears the accumulators for the next block
-    auto store_block = [&](int cb, int r0, f32x4 (&acc)[4]) {
-        const int col = cb * kAnyTile + 4 * n;
+    f32x4 acc[RT][4 * CG];
+    auto clear = [&]() {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = r0 + 16 * wave + 4 * q + i;
-            if (row < M && col < N) {
-                uint16_t *p = os + (int64_t)row * N + col;
-                if (col + 4 <= N) {
-                    *reinterpret_cast<u32x2_unaligned *>(p) =
-                        u32x2{Elem<DT>::pack2(acc[0][i], acc[1][i]), Elem<DT>::pack2(acc[2][i], acc[3][i])};
-                } else {
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-                    for (int t = 0; t < 3; ++t)
-                        if (col + t < N) p[t] = Elem<DT>::from_float(acc[t][i]);
-                }
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < 4; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < 4 * CG; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
     };
-    const int rounds = (M + kAnyTile - 1) / kAnyTile;
-    const int ncb = (N + kAnyTile - 1) / kAnyTile;
-    const int steps = ncb * nkc;                     // (column block, chunk) pairs of one round, chunk fastest
-    for (int round = first_round; round < rounds; round += round_step) {
-        const int r0 = round * kAnyTile;
-        f32x4 acc[4];
+    // lane (n, q): rows 16 (RT wave + rt) + 4 q + i, columns kCols cb + kLaneCols n .. of the block, side by side: one
+    // 8- or 16-byte store per row, the sixteen lanes of a row group writing 128 or 256 contiguous bytes; clears the
+    // accumulators
+    constexpr int kLaneCols = 4 * CG;
+    auto store_block = [&](int cb, int r0) __attribute__((always_inline)) {
+        const bool whole = r0 + kRows <= M && (cb + 1) * kCols <= N;       // no row or column of the block is outside
+        const int col = cb * kCols + kLaneCols * n;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        Line16 nx, ny;
-        if (steps > 0) {
-            nx = fetch_chunk16(resX, t1, M, K, r0, 0, tid);
-            ny = fetch_chunk16(resY, t2, N, K, 0, 0, tid);
-        }
-        int cb = 0, kc = 0;
-        for (int step = 0; step < steps; ++step) {
-            __syncthreads();                                           // the previous chunk is consumed
-            put_chunk16<false>(nx, t1, M, K, r0, kc * kAnyTile, sX, tid);
-            put_chunk16<true>(ny, t2, N, K, cb * kAnyTile, kc * kAnyTile, sY, tid);
-            int cb2 = cb, kc2 = kc + 1;
-            if (kc2 == nkc) { kc2 = 0; ++cb2; }
-            if (step + 1 < steps) {                                    // in flight under the matrix instructions
-                nx = fetch_chunk16(resX, t1, M, K, r0, kc2 * kAnyTile, tid);
-                ny = fetch_chunk16(resY, t2, N, K, cb2 * kAnyTile, kc2 * kAnyTile, tid);
-            }
-            __syncthreads();
+        for (int rt = 0; rt < RT; ++rt) {
+            uint16_t *p0 = os + (int64_t)(r0 + 16 * (RT * wave + rt) + 4 * q) * N + col;
 #pragma unroll
-            for (int ks = 0; ks < kAnyTile / 32; ++ks) {
-                const u32x4 av = t1 ? lds_tr8(xt + ks * 32 * kAnyPitch) : *reinterpret_cast<const u32x4 *>(xa + ks * 64);
+            for (int i = 0; i < 4; ++i) {
+                const int row = r0 + 16 * (RT * wave + rt) + 4 * q + i;
+                uint16_t *p = p0 + (int64_t)i * N;
+                if (whole || (row < M && col + kLaneCols <= N)) {
+                    if constexpr (CG == 2) {
+                        *reinterpret_cast<u32x4_unaligned *>(p) =
+                            u32x4{Elem<DT>::pack2(acc[rt][0][i], acc[rt][1][i]), Elem<DT>::pack2(acc[rt][2][i], acc[rt][3][i]),
+                                  Elem<DT>::pack2(acc[rt][4][i], acc[rt][5][i]), Elem<DT>::pack2(acc[rt][6][i], acc[rt][7][i])};
+                    } else {
+                        *reinterpret_cast<u32x2_unaligned *>(p) =
+                            u32x2{Elem<DT>::pack2(acc[rt][0][i], acc[rt][1][i]), Elem<DT>::pack2(acc[rt][2][i], acc[rt][3][i])};
+                    }
+                } else if (row < M) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const u32x4 bv = t2 ? lds_tr8(yt + ks * 32 * kAnyPitch + 32 * t)
-                                        : *reinterpret_cast<const u32x4 *>(ya + t * kAnyPitch + ks * 64);
-                    acc[t] = Elem<DT>::mfma(av, bv, acc[t]);
+                    for (int t = 0; t < kLaneCols - 1; ++t)
+                        if (col + t < N) p[t] = Elem<DT>::from_float(acc[rt][t][i]);
                 }
             }
-            if (kc == nkc - 1) store_block(cb, r0, acc);
-            cb = cb2; kc = kc2;
+        }
+        clear();
+    };
+    const int rounds = (M + kRows - 1) / kRows;
+    const int ncb = (N + kCols - 1) / kCols;
+    const int steps = ncb * nkc;                     // (column block, chunk) pairs of one round, chunk fastest
+    // With at most two chunks of k (K <= 128) the X chunks of a round stay in LDS, one per buffer, and are fetched
+    // once instead of once per column block; only Y streams.
+    const bool x_once = nkc <= 2;
+    for (int round = first_round; round < rounds; round += round_step) {
+        const int r0 = round * kRows;
+        clear();
+        // a stage = the registers of one chunk in flight (plain vectors: the staging union only lives inside the calls)
+        struct Stage { u32x4 x[RT][2], y[CG][2]; };
+        auto fetch = [&](Stage &st, int cb, int kc) __attribute__((always_inline)) {
+            if (!x_once || cb == 0) {
+#pragma unroll
+                for (int i = 0; i < RT; ++i) {
+                    const Line16 l = fetch_chunk16<4 * RT>(resX, t1, M, K, r0, kc * kAnyTile, tid + kAnyThreads * i);
+                    st.x[i][0] = l.v[0]; st.x[i][1] = l.v[1];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < CG; ++i) {
+                const Line16 l = fetch_chunk16<4 * CG>(resY, t2, N, K, cb * kCols, kc * kAnyTile, tid + kAnyThreads * i);
+                st.y[i][0] = l.v[0]; st.y[i][1] = l.v[1];
+            }
+        };
+        int f_cb = 0, f_kc = 0;                       // the chunk the next fetch takes
+        auto advance = [&]() {
+            if (++f_kc == nkc) { f_kc = 0; ++f_cb; }
+        };
+        Stage sa, sb;
+        if (steps > 0) { fetch(sa, f_cb, f_kc); advance(); }
+        if (steps > 1) { fetch(sb, f_cb, f_kc); advance(); }
+        int cb = 0, kc = 0;                           // the chunk being computed
+        auto do_step = [&](int step, Stage &st) __attribute__((always_inline)) {
+            unsigned char *buf = any_lds + (step & 1) * kBufBytes;
+            unsigned char *xbuf = any_lds + (x_once ? kc : step & 1) * kBufBytes;
+            if (!x_once || cb == 0) {
+#pragma unroll
+                for (int i = 0; i < RT; ++i) {
+                    Line16 l;
+                    l.v[0] = st.x[i][0]; l.v[1] = st.x[i][1];
+                    put_chunk16<false, 4 * RT, kPitchXT>(l, t1, M, K, r0, kc * kAnyTile, xbuf, tid + kAnyThreads * i);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < CG; ++i) {
+                Line16 l;
+                l.v[0] = st.y[i][0]; l.v[1] = st.y[i][1];
+                put_chunk16<true, 4 * CG, kPitchYT>(l, t2, N, K, cb * kCols, kc * kAnyTile, buf + AnyBuf<kRows>::bytes,
+                                                    tid + kAnyThreads * i);
+            }
+            if (step + 2 < steps) { fetch(st, f_cb, f_kc); advance(); }   // in flight under two steps of matrix instructions
+            // every wavefront has written its part of this chunk, and is done reading the chunk before last,
+            // whose buffer the NEXT step's writes go to
+            lds_barrier();
+            // the B operands are read two tiles ahead of the matrix instructions that use them (an LDS round trip
+            // is several times a matrix instruction), the A operands of the second k-step while the first computes
+            constexpr int kTiles = 4 * CG, kFrags = (kAnyTile / 32) * kTiles;
+            auto read_a = [&](int ks, int rt) __attribute__((always_inline)) {
+                return t1 ? lds_tr8<kPitchXT>(xbuf + xt + 32 * rt + ks * 32 * kPitchXT)
+                          : *reinterpret_cast<const u32x4 *>(xbuf + xa + 16 * rt * kAnyPitch + ks * 64);
+            };
+            auto read_b = [&](int f) __attribute__((always_inline)) {
+                const int ks = f / kTiles, t = f % kTiles;
+                return t2 ? lds_tr8<kPitchYT>(buf + yt + ks * 32 * kPitchYT + 32 * t)
+                          : *reinterpret_cast<const u32x4 *>(buf + ya + t * kAnyPitch + ks * 64);
+            };
+            u32x4 av[2][RT], bq[3];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) av[0][rt] = read_a(0, rt);
+            bq[0] = read_b(0);
+            bq[1] = read_b(1);
+#pragma unroll
+            for (int f = 0; f < kFrags; ++f) {
+                const int ks = f / kTiles, t = f % kTiles;
+                if (f + 2 < kFrags) bq[(f + 2) % 3] = read_b(f + 2);
+                if (t == 0 && ks + 1 < kAnyTile / 32) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) av[(ks + 1) & 1][rt] = read_a(ks + 1, rt);
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) acc[rt][t] = Elem<DT>::mfma(av[ks & 1][rt], bq[f % 3], acc[rt][t]);
+            }
+            if (kc == nkc - 1) store_block(cb, r0);
+            if (++kc == nkc) { kc = 0; ++cb; }
+        };
+        for (int step = 0; step < steps; step += 2) {
+            do_step(step, sa);
+            if (step + 1 < steps) do_step(step + 1, sb);
         }
         if (nkc == 0)                                                  // K = 0: the result is zeros
-            for (int c = 0; c < ncb; ++c) store_block(c, r0, acc);
+            for (int c = 0; c < ncb; ++c) store_block(c, r0);
+        if (round + round_step < rounds) lds_barrier();                // the next round's first chunk may take either buffer
     }
+}
+
+template <int DT, int RT, int CG, bool T1, bool T2>
+static void launch_any_build(const RunArgs &run, dim3 grid, hipStream_t stream) {
+    constexpr int kLds = 2 * (AnyBuf<kAnyTile * RT>::bytes + AnyBuf<kAnyTile * CG>::bytes);
+    if constexpr (kLds > 65536) {
+        static const bool attr_set = [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_any16_kernel<DT, RT, CG, T1, T2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds) == hipSuccess;
+        }();
+        (void)attr_set;
+    }
+    hipLaunchKernelGGL((gemm_any16_kernel<DT, RT, CG, T1, T2>), grid, dim3(kAnyThreads), kLds, stream, run);
+}
+template <int DT, int RT, int CG>
+static void launch_any(const RunArgs &run, dim3 grid, hipStream_t stream) {
+    const bool t1 = run.flags & kFlagTranspose1, t2 = run.flags & kFlagTranspose2;
+    if (t1 && t2) launch_any_build<DT, RT, CG, true, true>(run, grid, stream);
+    else if (t1) launch_any_build<DT, RT, CG, true, false>(run, grid, stream);
+    else if (t2) launch_any_build<DT, RT, CG, false, true>(run, grid, stream);
+    else launch_any_build<DT, RT, CG, false, false>(run, grid, stream);
 }
 
 int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream) {
@@ -228,18 +374,31 @@ int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_pla
     if (nseg <= 0) return BA_OK;
     RunArgs run = args;
     dim3 grid;
-    const int64_t items = info ? (int64_t)info->att_blocks64 * args.H : 0;
-    if (info && items < (int64_t(1) << 31)) {
+    // 128 x 128 steps where the segments are tall (four 64-row rounds per segment on average): half the operand
+    // traffic per result and 16-byte stores; batches of short segments finish in one or two steps per workgroup
+    // either way and do better with twice as many, smaller workgroups resident.  Measured, operands stored K x M and
+    // K x N, 128 / 64: 16 segments x 16 heads of 1024..4096 rows 1660 / 2120 us; 512 segments of 16..256 rows
+    // 24.0 / 20.5 us; 1024 segments, power-law sizes, 85 / 53 us.  BLOCKEDATTN_ANY_TILE=64|128 forces one.
+    static const int tile_env = [] { const char *e = getenv("BLOCKEDATTN_ANY_TILE"); return e ? atoi(e) : 0; }();
+    const bool big = tile_env ? tile_env == 128 : info && (int64_t)info->att_blocks64 >= 4 * (int64_t)info->nseg;
+    const int64_t items = info ? (int64_t)(big ? info->att_blocks128 : info->att_blocks64) * args.H : 0;
+    if (info && items < (int64_t(1) << 31) - 1024) {
         if (items == 0) return BA_OK;                   // no segment has rows
         run.ride_slots = 1;
-        grid = dim3((unsigned)items);
+        const int64_t unit = (int64_t)kDies * kAnyDieBlock;           // whole blocks for every die
+        grid = dim3((unsigned)((items + unit - 1) / unit * unit));
     } else {
         const bool head_fast = nseg <= 65535;           // segments then ride on gridDim.y
         if (head_fast) run.flags |= kFlagHeadFast;
         grid = head_fast ? dim3((unsigned)args.H, (unsigned)nseg, 4u) : dim3((unsigned)nseg, (unsigned)args.H, 4u);
     }
-    if (dtype == BA_F16) hipLaunchKernelGGL(gemm_any16_kernel<0>, grid, dim3(kAnyThreads), 0, stream, run);
-    else hipLaunchKernelGGL(gemm_any16_kernel<1>, grid, dim3(kAnyThreads), 0, stream, run);
+    if (dtype == BA_F16) {
+        if (big) launch_any<0, 2, 2>(run, grid, stream);
+        else launch_any<0, 1, 1>(run, grid, stream);
+    } else {
+        if (big) launch_any<1, 2, 2>(run, grid, stream);
+        else launch_any<1, 1, 1>(run, grid, stream);
+    }
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 

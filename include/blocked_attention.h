@@ -243,6 +243,13 @@ int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg, int 
  * attributes (host-side calls that do not belong in a stream capture): make
  * one call per device outside any capture, with any small batch, before the
  * calls that are captured.
+ * Small batches (at most 512 segments, 1024 (segment, head) pairs and 2^24
+ * values in each of A + B and out; modes BA_META_FROM_LISTS and BA_META_GIVEN)
+ * run as ONE kernel launch that derives every segment's offsets and class from
+ * the metadata itself: no scheduler launch, and the buffer is not touched (what
+ * the reference does in host round trips at spBlkGEMM.cu:943-983 and 985-1033
+ * happens inside the compute kernel).  The results are those of the plan-driven
+ * kernels, except that tiny segments are not packed into shared tiles.
  * At most BA_STATIC_MAX_SEGMENTS segments: more returns BA_ERR_WORKSPACE.
  * All calls on one GPU share that GPU's buffer: calls that overlap on one GPU
  * (different streams or threads) race; calls on one stream do not.

@@ -5,7 +5,7 @@ import torch
 
 import oracle
 from blockedattention_amd import capi, workloads
-from _util import assert_scores_close, make_plan, random_operands, run_all
+from _util import assert_scores_close, dev_i64, make_plan, random_operands, run_all
 
 pytestmark = pytest.mark.gpu
 
@@ -123,6 +123,35 @@ def test_gapped_prefix_sums_given_with_lists(dev):
         ref = A[:, o1:o1 + m * k].float().reshape(2, m, k) @ B[:, o2:o2 + n * k].float().reshape(2, n, k).transpose(1, 2)
         assert_scores_close(o[:, oo:oo + m * n], ref.reshape(2, -1), "gapped")
     assert (o[:, 24:30] == 9.0).all()                          # the gap is never written
+
+
+def test_gapped_prefix_sums_with_a_transposed_operand(dev):
+    # the any-layout 16-bit kernel behind caller-given prefix sums with holes in all three tensors: B_g stored K x N
+    # (and then both operands k-major); the holes of the output keep what they held
+    rng = np.random.default_rng(17)
+    n = 9
+    M = rng.integers(1, 150, n).astype(np.int64); N = rng.integers(1, 200, n).astype(np.int64)
+    K = rng.choice([8, 24, 40, 64, 100, 136], n).astype(np.int64)
+    gap = rng.integers(1, 4, n).astype(np.int64) * 3            # odd holes: later segments start at odd elements
+    start = lambda area: np.concatenate([[0], np.cumsum(area + gap)]).astype(np.int64)
+    a1, a2, ao = start(M * K), start(N * K), start(M * N)
+    H = 2
+    g = torch.Generator().manual_seed(4)
+    A = torch.randn((H, int(a1[-1])), generator=g).half(); B = torch.randn((H, int(a2[-1])), generator=g).half()
+    plan = capi.plan_gemm(n, dev, dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev), dev_i64(a1, dev), dev_i64(a2, dev),
+                          dev_i64(ao, dev), mode=capi.META_GIVEN)
+    plan.read()
+    for t1, t2 in ((False, True), (True, True)):
+        out = torch.full((H, int(ao[-1])), 9.0, dtype=torch.float16, device=dev)
+        capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, H, int(a1[-1]), int(a2[-1]), int(ao[-1]), t1, t2)
+        o = out.float().cpu()
+        for i in range(n):
+            m, nn, k = int(M[i]), int(N[i]), int(K[i])
+            a = A[:, a1[i]:a1[i] + m * k].float(); b = B[:, a2[i]:a2[i] + nn * k].float()
+            a = a.reshape(H, k, m).transpose(1, 2) if t1 else a.reshape(H, m, k)
+            b = b.reshape(H, k, nn) if t2 else b.reshape(H, nn, k).transpose(1, 2)
+            assert_scores_close(o[:, ao[i]:ao[i] + m * nn], (a @ b).reshape(H, -1), f"segment {i}, transposes {t1} {t2}")
+            assert (o[:, ao[i] + m * nn:ao[i + 1]] == 9.0).all(), f"the hole behind segment {i} was written"
 
 
 def test_many_tiny_segments_are_packed(dev):
