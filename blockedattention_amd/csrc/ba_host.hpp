@@ -17,7 +17,8 @@ enum RunFlags : int {
     kFlagTilesToo = 32,    // strip kernel, 64 KiB launch: further blocks run the tile kernel's workgroups (tile_zdim, tile_groups)
     kFlagQuiet = 64,       // an earlier launch of the same call reports a plan that does not match
     kFlagSmallToo = 128,   // strip kernel, 64 KiB launch: the slots from both_split on walk the main launch's list
-    kFlagHeadFast = 256    // strip kernel: grid (head, slot, z) instead of (slot, head, z)
+    kFlagHeadFast = 256,   // strip kernel: grid (head, slot, z) instead of (slot, head, z)
+    kFlagPipeToo = 512     // tile kernel: the pipelined row-block kernel runs in the same call and takes its segments
 };
 
 struct RunArgs {

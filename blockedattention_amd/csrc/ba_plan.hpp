@@ -66,7 +66,8 @@ enum PrefixKind {
     kPfxAtt64 = 12,   // GEMM plans: ceil(M/64) for every segment with rows (one-pass attention, any-layout GEMM)
     kPfxAtt128 = 13,  // the same in row blocks of 128
     kPfxMini = 14,    // 1 for a segment of the strip kernel's main list that is small enough for one wavefront
-    kNumPrefix = 15
+    kPfxPipe = 15,    // 1 for a segment of the tile list that the pipelined row-block kernel can take (fused call)
+    kNumPrefix = 16
 };
 
 // "Mini" segments: strip-class segments of at most 64 rows whose B_g needs at most kMiniBlocks LDS blocks and at most
@@ -103,7 +104,9 @@ struct PlanHeader {
     int32_t small_max_N, small_max_M;   // maxima over the segments of the strip kernel's main launch
     int32_t att_blocks64, att_blocks128;   // totals of kPfxAtt64 / kPfxAtt128: the one-pass attention's row blocks per head
     int32_t mini_count;      // total of kPfxMini
-    int32_t pad_[18];
+    int32_t pipe_count;      // total of kPfxPipe
+    int32_t pipe_groups;     // bumped by every workgroup of the pipelined row-block kernel that found work in this plan
+    int32_t pad_[16];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 
@@ -126,6 +129,13 @@ constexpr int kTileCols = 128;
 __host__ __device__ inline bool tile_segment(int kind, int N, int K) {
     if (kind == kSegSplit || kind == kSegWide) return true;
     return kind == kSegStrip && !fast_strip_shape(N, K) && N >= kTileCols;
+}
+
+// Segments of the tile list that the pipelined row-block kernel takes in a fused call with 16-bit results: the A
+// fragments of a wavefront's 64 rows stay in registers (K <= 128) and the chunk pipeline is four chunks of 64
+// columns deep.
+__host__ __device__ inline bool pipe_segment(int kind, int N, int K) {
+    return tile_segment(kind, N, K) && K <= 128 && N > 3 * 64;
 }
 
 // Launch class (work list) of a segment of a GEMM plan, or -1 for none.

@@ -124,6 +124,8 @@ static int info_from_header(const PlanHeader &h, ba_plan_info *info) {
     info->att_blocks64 = h.att_blocks64;
     info->att_blocks128 = h.att_blocks128;
     info->list_mini = h.mini_count;
+    info->list_pipe = h.pipe_count;
+    info->pipe_groups = h.pipe_groups;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 

@@ -125,16 +125,14 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     }
     bool valid;
     const Seg s = load_listed(pv, entry, h, a, valid);
-    if (!valid || !tile_segment(s.kind, s.N, s.K)) return;
+    if (!valid || !pipe_segment(s.kind, s.N, s.K)) return;      // (the tile kernel of the same call takes the others)
     const int M = s.M, N = s.N, K = s.K;
     const int nrb = (M + kRpBlockRows - 1) / kRpBlockRows;
     const int b_begin = (int)((int64_t)z0 * nrb / zdim), b_end = (int)((int64_t)(z0 + 1) * nrb / zdim);
     if (b_begin >= b_end) return;
     const int ncb = (N + kRpCols - 1) / kRpCols;
-    if (K > 128 || ncb < kRpStages) {            // the launch was sized for another plan
-        if (z0 == 0 && threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
-        return;
-    }
+    static_assert(kRpStages == 4 && kRpCols == 64, "pipe_segment() admits segments of at least four chunks");
+    if (threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->pipe_groups, 1);
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int set = wave >> 2, wq = wave & 3;
@@ -610,10 +608,16 @@ static int launch_rp(const RunArgs &args, unsigned groups, int zdim, int weave, 
 }
 
 // Launches the pipelined row-block kernel over (list entry, head, share of the row blocks): the fused pair for
-// large segments with K <= 128 and 16-bit results.  Needs the plan summary.
+// large segments with K <= 128 and 16-bit results.  `slots` = entries of the tile list (with the plan summary) or
+// the segment count (without: the workgroups behind the list's end leave at once); the kernel takes the entries
+// that pipe_segment() admits and leaves the others to the tile kernel.
 int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_info *info, hipStream_t stream) {
-    if (!info || info->max_K > 128 || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
+    if (args.flags & kFlagOutF32) return BA_ERR_UNSUPPORTED;
     if (slots <= 0) return BA_OK;
+    // Without the summary every (segment, head) gets a workgroup that may find nothing, and a workgroup of this kernel
+    // holds a whole compute unit while it looks (1024 segments x 4 heads of small segments: + 40 us): only for small
+    // batches, where large segments are likely and the empty workgroups are few.
+    if (!info && slots * args.H > 1024) return BA_ERR_UNSUPPORTED;
     int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
     static const int forced_z = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE_Z"); return e ? atoi(e) : 0; }();
     static const int forced_w = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE_WEAVE"); return e ? atoi(e) : 0; }();
@@ -624,7 +628,8 @@ int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_
     // per compute unit with an equal share of all the work (contiguous runs of pairs and row blocks): 1744 .. 1906 us,
     // the dies with the narrow pairs finishing last.  BLOCKEDATTN_ROWPIPE_Z and _WEAVE override.
     const int cus = device_cu_count();
-    const int64_t z_max = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRpBlockRows - 1) / kRpBlockRows));
+    // (without the summary the tallest segment is unknown: up to eight shares, which a short segment leaves empty)
+    const int64_t z_max = !info ? 8 : std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kRpBlockRows - 1) / kRpBlockRows));
     int64_t z = std::min<int64_t>(z_max, std::max<int64_t>(1, (2 * (int64_t)cus + pairs - 1) / pairs));
     if (forced_z > 0) z = std::min<int64_t>(z_max, forced_z);
     const int64_t weave = std::max<int64_t>(1, std::min<int64_t>(forced_w > 0 ? forced_w : 1, pairs / kDies));

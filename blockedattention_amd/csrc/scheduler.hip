@@ -230,6 +230,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
 #pragma unroll
         for (int q = 0; q < kNumLists; ++q) v32[q] = (cls == q && !mini) ? 1 : 0;
         v32[kPfxMini] = mini ? 1 : 0;
+        v32[kPfxPipe] = (cls == kListTile && pipe_segment(seg_kind, ni, ki)) ? 1 : 0;
         const bool wide_rows = mi >= 1 && ni > kRunCols;      // the softmax row kernel's, whatever the plan kind
         v32[kListRows] = wide_rows ? 1 : 0;
         weight += max((int64_t)mi, (int64_t)strips * chunks) + 1;
@@ -354,6 +355,8 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->att_blocks64 = base32[kPfxAtt64];
         h->att_blocks128 = base32[kPfxAtt128];
         h->mini_count = base32[kPfxMini];
+        h->pipe_count = base32[kPfxPipe];
+        h->pipe_groups = 0;
         plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
         plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
         if (a.mailbox) {

@@ -385,6 +385,7 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
     if (!valid) return;
     const int kind = s.kind;
     if (!tile_segment(kind, s.N, s.K)) return;
+    if ((a.flags & kFlagPipeToo) && pipe_segment(kind, s.N, s.K)) return;      // the other kernel of this call takes it
     tile_rows<DT, FUSED, F32OUT>(a, s, z0, zdim, lds);
 }
 

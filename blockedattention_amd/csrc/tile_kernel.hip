@@ -21,24 +21,40 @@ static void launch_one(const RunArgs &args, unsigned groups, int zdim, hipStream
 int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                  hipStream_t stream) {
     static const int use_rowblocks = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK"); return e ? atoi(e) : 1; }();
-    if (use_rowblocks && info && info->max_K <= 128 && !(args.flags & kFlagOutF32))
+    if (slots <= 0) return BA_OK;
+    RunArgs targs = args;
+    if (use_rowblocks && fused && !(args.flags & kFlagOutF32)) {
+        // The fused pair with 16-bit results: every segment with K <= 128 goes to the pipelined row-block kernel,
+        // the others stay here.  The plan counts the former (list_pipe); without the summary both kernels are
+        // launched over the whole list and each workgroup keeps to its own kind of segment.
+        const int64_t pipe = info ? info->list_pipe : slots;
+        if (pipe > 0) {
+            const int st = launch_rowpipe(dtype, args, slots, info, stream);
+            if (st == BA_OK) {
+                if (info && pipe >= slots) return BA_OK;          // nothing left for the tile kernel
+                targs.flags |= kFlagPipeToo | kFlagQuiet;
+            } else if (st != BA_ERR_UNSUPPORTED) {
+                return st;
+            }
+        }
+    } else if (use_rowblocks && !fused && info && info->max_K <= 128) {
         return launch_rowblocks(dtype, fused, args, slots, info, stream);
+    }
     int64_t z = 4;
     if (info)
         z = std::max<int64_t>(1, std::min<int64_t>(64, (std::max<int64_t>(info->max_M, 1) + kTileRows - 1) / kTileRows));
-    if (slots <= 0) return BA_OK;
     const int64_t pairs = (slots + kDies - 1) / kDies * kDies * args.H;   // entries padded to whole dies
     const int64_t groups = pairs * z;
     if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
     const bool f32out = args.flags & kFlagOutF32;
     if (dtype == BA_F16) {
-        if (!fused) launch_one<0, false, false>(args, (unsigned)groups, (int)z, stream);
-        else if (f32out) launch_one<0, true, true>(args, (unsigned)groups, (int)z, stream);
-        else launch_one<0, true, false>(args, (unsigned)groups, (int)z, stream);
+        if (!fused) launch_one<0, false, false>(targs, (unsigned)groups, (int)z, stream);
+        else if (f32out) launch_one<0, true, true>(targs, (unsigned)groups, (int)z, stream);
+        else launch_one<0, true, false>(targs, (unsigned)groups, (int)z, stream);
     } else if (dtype == BA_BF16) {
-        if (!fused) launch_one<1, false, false>(args, (unsigned)groups, (int)z, stream);
-        else if (f32out) launch_one<1, true, true>(args, (unsigned)groups, (int)z, stream);
-        else launch_one<1, true, false>(args, (unsigned)groups, (int)z, stream);
+        if (!fused) launch_one<1, false, false>(targs, (unsigned)groups, (int)z, stream);
+        else if (f32out) launch_one<1, true, true>(targs, (unsigned)groups, (int)z, stream);
+        else launch_one<1, true, false>(targs, (unsigned)groups, (int)z, stream);
     } else {
         return BA_ERR_UNSUPPORTED;
     }

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BA_ABI_VERSION 4
+#define BA_ABI_VERSION 5
 
 typedef void *ba_stream_t; /* hipStream_t */
 
@@ -86,6 +86,10 @@ typedef struct ba_plan_info {
     /* segments of the strip kernel's main launch that one wavefront can take alone (at most 64 rows, B_g of
      * at most 16 KiB); list_small counts the others */
     int32_t list_mini;
+    /* segments of list_tile that the pipelined row-block kernel takes in a fused call with 16-bit results
+     * (K <= 128), and how many workgroups of that kernel have found work in this plan since it was built */
+    int32_t list_pipe;
+    int32_t pipe_groups;
 } ba_plan_info;
 
 const char *ba_status_string(int status);

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = capi.load()
     for name in declared_symbols():
         assert hasattr(lib, name), name
-    assert lib.ba_abi_version() == 4
+    assert lib.ba_abi_version() == 5
 
 
 def test_plan_bytes_and_status_strings():

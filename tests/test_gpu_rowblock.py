@@ -133,3 +133,43 @@ def test_k_zero_in_the_tile_kernel(dev):
     # has no operand bytes there either, and the rows are zeros (product) or 1/N (fused pair)
     run_all(dev, [40, 200, 70], [300, 130, 260], [0, 0, 64], 2, torch.float16, 0.2, summary=False)
     run_all(dev, [40, 200, 70], [300, 130, 260], [0, 0, 136], 2, torch.bfloat16, 0.2)
+
+
+def fused_only(dev, M, N, K, H, dtype, scale, summary, seed=0, out_dtype=None):
+    M = np.asarray(M, np.int64); N = np.asarray(N, np.int64); K = np.asarray(K, np.int64)
+    A, B = random_operands(M, N, K, H, dtype, seed)
+    plan = make_plan(dev, M, N, K, read=summary)
+    d1, d2, do = int((M * K).sum()), int((N * K).sum()), int((M * N).sum())
+    out = torch.full((H, do), float("nan"), dtype=out_dtype or dtype, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, H, d1, d2, do, scale)
+    assert_probs_close(out, oracle.per_segment_torch(A, B, M, N, K, scale), "fused")
+    info = plan.read()
+    assert info.run_errors == 0
+    return info
+
+
+def test_the_pipelined_kernel_is_chosen_segment_by_segment(dev):
+    # K = 136, 160 and 256 keep a segment in the tile kernel; its neighbours with K <= 128 still take the pipelined
+    # row-block kernel, in the same call (the plan counts them, the kernel counts the workgroups that worked)
+    M = [300, 520, 100, 260, 700, 64]; N = [400, 300, 1000, 263, 513, 200]; K = [128, 136, 64, 160, 8, 256]
+    for dtype in (torch.float16, torch.bfloat16):
+        info = fused_only(dev, M, N, K, 2, dtype, 0.13, summary=True, seed=3)
+        assert info.list_tile == 6 and info.list_pipe == 3
+        assert info.pipe_groups >= 3 * 2                      # at least one workgroup per eligible segment and head
+
+
+def test_the_pipelined_kernel_runs_without_the_host_summary(dev):
+    # no summary was read between scheduler and kernels (graph replays, the one-call entry point): the large
+    # segments with K <= 128 still go through the pipelined kernel, the others through the tile kernel
+    M = [300, 520, 1030, 260]; N = [400, 300, 1000, 263]; K = [128, 136, 64, 96]
+    info = fused_only(dev, M, N, K, 3, torch.bfloat16, 0.2, summary=False, seed=5)
+    assert info.list_pipe == 3 and info.pipe_groups >= 3 * 3
+    # all of them eligible: the tile kernel is still launched (nothing told the host) and finds nothing
+    info = fused_only(dev, M[:1] + M[2:], N[:1] + N[2:], K[:1] + K[2:], 2, torch.float16, 0.2, summary=False, seed=6)
+    assert info.list_pipe == 3 and info.pipe_groups >= 3 * 2
+
+
+def test_fp32_probabilities_of_large_segments_stay_in_the_tile_kernel(dev):
+    info = fused_only(dev, [300, 260], [400, 263], [128, 96], 2, torch.bfloat16, 0.2, summary=True, seed=7,
+                      out_dtype=torch.float32)
+    assert info.list_pipe == 2 and info.pipe_groups == 0

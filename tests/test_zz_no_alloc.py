@@ -46,7 +46,8 @@ def test_two_calls_in_a_row_the_second_smaller(dev):
     rng = np.random.default_rng(5)
     n = 640                                                 # beyond the one-launch path: scheduler, plan buffer, kernels
     M = rng.integers(1, 90, n); N = rng.integers(1, 200, n); K = rng.choice(np.arange(8, 129, 8), n)
-    N[7] = 700; M[7] = 150; K[7] = 128                   # one segment of the tile kernel
+    N[7] = 700; M[7] = 150; K[7] = 136                   # one segment of the tile kernel (in every batch below)
+    N[520] = 600; M[520] = 300; K[520] = 128             # and one of the pipelined row-block kernel (in the two large ones)
     both_ways(dev, M, N, K, 3, torch.bfloat16, 0.11, seed=1)
     both_ways(dev, M[:530], N[:530], K[:530], 2, torch.float16, 0.2, seed=2)   # smaller batch into the same buffer
     both_ways(dev, M[:40], N[:40], K[:40], 2, torch.float16, 0.2, seed=2)      # small enough for the single launch
