@@ -562,8 +562,6 @@ int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, c
                      hipStream_t stream) {
     if (!info || info->max_K > 128 || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
     if (slots <= 0) return BA_OK;
-    static const int use_pipe = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE"); return e ? atoi(e) : 1; }();
-    if (fused && use_pipe) return launch_rowpipe(dtype, args, slots, info, stream);
     int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
     // Workgroups per pair Z (workgroup z of a pair takes its row blocks z, z + Z, ..) and pairs of a die that take
     // turns in the grid.  Sixteen workgroups of one pair that start together fetch the same lines of B_g at the same

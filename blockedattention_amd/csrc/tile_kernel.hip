@@ -23,7 +23,10 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
     static const int use_rowblocks = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK"); return e ? atoi(e) : 1; }();
     if (slots <= 0) return BA_OK;
     RunArgs targs = args;
-    if (use_rowblocks && fused && !(args.flags & kFlagOutF32)) {
+    static const int use_pipe = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE"); return e ? atoi(e) : 1; }();
+    if (use_rowblocks && fused && !use_pipe && info && info->max_K <= 128 && !(args.flags & kFlagOutF32))
+        return launch_rowblocks(dtype, fused, args, slots, info, stream);     // the kernel before the pipelined one
+    if (use_rowblocks && fused && use_pipe && !(args.flags & kFlagOutF32)) {
         // The fused pair with 16-bit results: every segment with K <= 128 goes to the pipelined row-block kernel,
         // the others stay here.  The plan counts the former (list_pipe); without the summary both kernels are
         // launched over the whole list and each workgroup keeps to its own kind of segment.
