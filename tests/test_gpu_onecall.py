@@ -189,3 +189,42 @@ def test_graph_replays_follow_the_lists(dev):
         assert_probs_close(out, oracle.per_segment_torch(Ah, Bh, m, m, K, scale), f"replay {replay}")
         assert torch.equal(acc[2].cpu(), torch.as_tensor(oracle.lists_to_accum(m, m, K)[2]))
         assert float(junk) == float(junk)
+
+
+def test_unaligned_base_pointer_takes_the_element_wise_rows(dev):
+    # A two bytes off a 16-byte boundary: no segment may use 16-byte operand loads, every workgroup walks its rows
+    rng = np.random.default_rng(41)
+    n = 30
+    M = rng.integers(1, 60, n).astype(np.int64); N = rng.integers(1, 300, n).astype(np.int64)
+    K = rng.choice(np.arange(8, 72, 8), n).astype(np.int64)
+    H = 2
+    A, B = random_operands(M, N, K, H, torch.float16, 8)
+    d1, d2, do = int((M * K).sum()), int((N * K).sum()), int((M * N).sum())
+    big = torch.zeros(H * d1 + 1, dtype=torch.float16, device=dev)
+    big[1:] = A.reshape(-1).to(dev)
+    out = torch.full((H, do), float("nan"), dtype=torch.float16, device=dev)
+    capi.gemm_softmax_static(dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev), big[1:], B.to(dev), out, H, d1, d2, do, 0.3)
+    torch.cuda.synchronize()
+    assert_probs_close(out, oracle.per_segment_torch(A, B, M, N, K, 0.3), "unaligned A")
+
+
+def test_given_prefix_sums_that_overlap_are_rejected(dev):
+    M = np.array([20, 30], np.int64); N = np.array([24, 36], np.int64); K = np.array([32, 32], np.int64)
+    a1 = np.array([0, 640, 1600], np.int64); a2 = np.array([0, 768, 1920], np.int64)
+    ao = np.array([0, 400, 1560], np.int64)                # segment 0 needs 480 results, its slot holds 400
+    A = torch.randn((1, 1600)).half(); B = torch.randn((1, 1920)).half()
+    out = torch.full((1, 1560), float("nan"), dtype=torch.float16, device=dev)
+    capi.gemm_softmax_static(dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev), A.to(dev), B.to(dev), out, 1, 1600, 1920, 1560,
+                             1.0, dev_i64(a1, dev), dev_i64(a2, dev), dev_i64(ao, dev), mode=capi.META_GIVEN)
+    torch.cuda.synchronize()
+    assert torch.isnan(out).all()
+
+
+def test_many_heads_up_to_the_pair_limit_and_beyond(dev):
+    # 200 segments x 5 heads = 1000 pairs: the single launch; x 6 heads: scheduler + plan-driven kernels; same results
+    rng = np.random.default_rng(43)
+    n = 200
+    M = rng.integers(1, 70, n).astype(np.int64); N = rng.integers(1, 130, n).astype(np.int64)
+    K = rng.choice(np.arange(8, 72, 8), n).astype(np.int64)
+    for H in (5, 6):
+        run_static(dev, M, N, K, H, torch.bfloat16, 0.21, seed=H)
