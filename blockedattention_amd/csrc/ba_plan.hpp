@@ -132,10 +132,10 @@ __host__ __device__ inline bool tile_segment(int kind, int N, int K) {
 }
 
 // Segments of the tile list that the pipelined row-block kernel takes in a fused call with 16-bit results: the A
-// fragments of a wavefront's 64 rows stay in registers (K <= 128) and the chunk pipeline is four chunks of 64
+// fragments of a wavefront's 64 rows stay in registers (K <= 128) and the chunk pipeline is five chunks of 64
 // columns deep.
 __host__ __device__ inline bool pipe_segment(int kind, int N, int K) {
-    return tile_segment(kind, N, K) && K <= 128 && N > 3 * 64;
+    return tile_segment(kind, N, K) && K <= 128 && N > 4 * 64;
 }
 
 // Launch class (work list) of a segment of a GEMM plan, or -1 for none.

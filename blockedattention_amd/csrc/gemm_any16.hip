@@ -234,12 +234,12 @@ __global__ __launch_bounds__(kAnyThreads, RT * CG >= 4 ? 2 : 4) void gemm_any16_
                 uint16_t *p = p0 + (int64_t)i * N;
                 if (whole || (row < M && col + kLaneCols <= N)) {
                     if constexpr (CG == 2) {
-                        *reinterpret_cast<u32x4_unaligned *>(p) =
-                            u32x4{Elem<DT>::pack2(acc[rt][0][i], acc[rt][1][i]), Elem<DT>::pack2(acc[rt][2][i], acc[rt][3][i]),
-                                  Elem<DT>::pack2(acc[rt][4][i], acc[rt][5][i]), Elem<DT>::pack2(acc[rt][6][i], acc[rt][7][i])};
+                        store_result<false>(reinterpret_cast<u32x4_unaligned *>(p),
+                                     u32x4{Elem<DT>::pack2(acc[rt][0][i], acc[rt][1][i]), Elem<DT>::pack2(acc[rt][2][i], acc[rt][3][i]),
+                                           Elem<DT>::pack2(acc[rt][4][i], acc[rt][5][i]), Elem<DT>::pack2(acc[rt][6][i], acc[rt][7][i])});
                     } else {
-                        *reinterpret_cast<u32x2_unaligned *>(p) =
-                            u32x2{Elem<DT>::pack2(acc[rt][0][i], acc[rt][1][i]), Elem<DT>::pack2(acc[rt][2][i], acc[rt][3][i])};
+                        store_result<false>(reinterpret_cast<u32x2_unaligned *>(p),
+                                     u32x2{Elem<DT>::pack2(acc[rt][0][i], acc[rt][1][i]), Elem<DT>::pack2(acc[rt][2][i], acc[rt][3][i])});
                     }
                 } else if (row < M) {
 #pragma unroll

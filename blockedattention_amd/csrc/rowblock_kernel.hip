@@ -282,7 +282,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
 #pragma unroll
                 for (int t = 2 * h; t < 2 * h + 2; ++t) {
                     const u32x4 v = ring_read16(rbase0 + t * 8 * kRingPitch, upos[t] ^ par);
-                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, v0[t] == kOutOfRange ? kOutOfRange : v0[t] + adv, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, v0[t] == kOutOfRange ? kOutOfRange : v0[t] + adv, 0, kResultAux);
                 }
                 asm volatile("" ::: "memory");
             };
@@ -301,11 +301,11 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                     const u32x4 v = ring_read16(rbase0 + t * 8 * kRingPitch, upos[t] ^ par);
                     const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRbCols * cbi;      // first column of the piece
                     const uint32_t voff = (col < 0 || col + 8 > N || v0[t] == kOutOfRange) ? kOutOfRange : v0[t] + adv;
-                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, kResultAux);
                 }
                 if (cbi == 0) {
                     const u32x4 v = *reinterpret_cast<const u32x4 *>(et_base);          // columns [0, 8)
-                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, kResultAux);
                 }
                 if (cbi == ncb - 1) {
                     // the window behind the last chunk (what is left of the rows), then columns [N-8, N)
@@ -315,10 +315,10 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                         const u32x4 v = ring_read16(rbase0 + t * 8 * kRingPitch, upos[t] ^ par2);
                         const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRbCols * ncb;
                         const uint32_t voff = (col + 8 <= N && v0[t] != kOutOfRange) ? v0[t] + 128u * (uint32_t)ncb : kOutOfRange;
-                        __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, kResultAux);
                     }
                     const u32x4 v = ring_read16(et_base, (2 * (N - 8)) & 255);
-                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off == kOutOfRange ? kOutOfRange : et_off + 2u * (uint32_t)(N - 8), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off == kOutOfRange ? kOutOfRange : et_off + 2u * (uint32_t)(N - 8), 0, kResultAux);
                 }
                 asm volatile("" ::: "memory");
             };

@@ -47,7 +47,10 @@ constexpr int kRpWaveRows = 16 * kRpRT;                   // 64
 constexpr int kRpBlockRows = kRpSetWaves * kRpWaveRows;   // 256 rows per set and step
 constexpr int kRpCols = 64;                               // columns per chunk
 constexpr int kRpStageBytes = kRpCols * 256;              // 16 KiB: 64 rows of B_g x 128 k
-constexpr int kRpStages = 4;
+#ifndef RP_STAGES
+#define RP_STAGES 5
+#endif
+constexpr int kRpStages = RP_STAGES;
 constexpr int kRpFillInsts = kRpStageBytes / 1024 / kRpSetWaves;   // global->LDS instructions per filling wavefront and chunk (4)
 constexpr int kRpStoreInsts = kRpWaveRows / 8;            // window stores per wavefront and chunk (8)
 constexpr int kRpRingPitch = 296;                         // 128 columns + a copy of the first 16 behind them; 74 words: the
@@ -55,12 +58,18 @@ constexpr int kRpRingPitch = 296;                         // 128 columns + a cop
 constexpr int kRpRingBytes = kRpWaveRows * kRpRingPitch;  // per wavefront of a set
 constexpr int kRpFlagOffset = kRpStages * kRpStageBytes + kRpSetWaves * kRpRingBytes;
 constexpr int kRpLdsBytes = kRpFlagOffset + 64;
+// Cache policy of the result stores: non-temporal.  The results are written once and never read by this kernel; as
+// ordinary stores they push the chunks of B_g, which every step reads again, out of the die's L2, and the fills then
+// wait behind the write stream (measured: the filling set waits 2500 cycles per iteration for its chunk with the
+// stores, 540 without them; 16 x 16 pairs of 1024..4096 rows and columns: 1490 us -> 1395 us with this bit).
+constexpr int kRpStoreAux = kResultAux;
 constexpr uint32_t kRpOutOfRange = 0x80000000u;           // byte offset no segment reaches (areas are below 2^31 bytes)
 
 enum RpRole : int { kRoleNone = 0, kRoleSum = 1, kRoleMax = 2, kRoleSumSafe = 3, kRoleOut = 4 };
 
-__device__ __forceinline__ void rp_wait_vm_upto(int n) {  // n in {0, 4, 8}, wave-uniform
-    if (n >= 8) wait_vm<8>();
+__device__ __forceinline__ void rp_wait_vm_upto(int n) {  // wave-uniform; the largest listed count not above n
+    if (n >= 12) wait_vm<12>();
+    else if (n >= 8) wait_vm<8>();
     else if (n >= 4) wait_vm<4>();
     else wait_vm<0>();
 }
@@ -131,7 +140,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     const int b_begin = (int)((int64_t)z0 * nrb / zdim), b_end = (int)((int64_t)(z0 + 1) * nrb / zdim);
     if (b_begin >= b_end) return;
     const int ncb = (N + kRpCols - 1) / kRpCols;
-    static_assert(kRpStages == 4 && kRpCols == 64, "pipe_segment() admits segments of at least four chunks");
+    static_assert(kRpStages <= 5 && kRpCols == 64, "pipe_segment() admits segments of at least five chunks");
     if (threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->pipe_groups, 1);
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
     const int wave = uniform((int)(threadIdx.x >> 6));
@@ -255,7 +264,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
     };
     auto ring_store = [&](int cbi, auto t_c) __attribute__((always_inline)) {
         constexpr int t = decltype(t_c)::value;
-        __builtin_amdgcn_raw_buffer_store_b128(ring_ld, out_res, v0[t] + 128u * (uint32_t)cbi, 0, 0);        // (the range check sees the vector offset only)
+        __builtin_amdgcn_raw_buffer_store_b128(ring_ld, out_res, v0[t] + 128u * (uint32_t)cbi, 0, kRpStoreAux);        // (the range check sees the vector offset only)
         asm volatile("" ::: "memory");
     };
     // First or last chunk: pieces before column 0 or past column N are dropped, and the end pieces the windows
@@ -272,11 +281,11 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             const u32x4 v = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ par);
             const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRpCols * cbi;      // first column of the piece
             const uint32_t voff = (col < 0 || col + 8 > N) ? kRpOutOfRange : v0[t] + adv;
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, kRpStoreAux);
         }
         if (cbi == 0) {
             const u32x4 v = rp_ring_read16(et_base, 0);                         // columns [0, 8)
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off, 0, kRpStoreAux);
         }
         if (cbi == ncb - 1) {
             // the window behind the last chunk (what is left of the rows), then columns [N-8, N)
@@ -286,10 +295,10 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
                 const u32x4 v = rp_ring_read16(lds + rbase_o + t * 8 * kRpRingPitch, upos[t] ^ par2);
                 const int col = (((upos[t] >> 1) + 64) & 127) - 64 + kRpCols * ncb;
                 const uint32_t voff = col + 8 <= N ? v0[t] + 128u * (uint32_t)ncb : kRpOutOfRange;
-                __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(v, out_res, voff, 0, kRpStoreAux);
             }
             const u32x4 v = rp_ring_read16(et_base, (2 * (N - 8)) & 255);
-            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off + 2u * (uint32_t)(N - 8), 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(v, out_res, et_off + 2u * (uint32_t)(N - 8), 0, kRpStoreAux);
         }
         asm volatile("" ::: "memory");
     };
@@ -493,15 +502,18 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
         int pf_cbi = 0, pf_stage = 0;
         auto sync = [&](int i, bool spread) __attribute__((always_inline)) {
             if (filler && i >= kRpStages - 1) {
-                int later = 2 * kRpFillInsts;
-                if (final_step) later = kRpFillInsts * ((i + 1 < ncb ? 1 : 0) + (i + 2 < ncb ? 1 : 0));
+                int later = (kRpStages - 2) * kRpFillInsts;
+                if (final_step) {
+                    later = 0;
+                    for (int d = 1; d <= kRpStages - 2; ++d) later += i + d < ncb ? kRpFillInsts : 0;
+                }
                 rp_wait_vm_upto(later);
             }
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             int cbi = i + kRpStages - 1;
             if (cbi >= ncb) cbi -= ncb;
             pf_cbi = cbi;
-            pf_stage = (gpos + i + kRpStages - 1) & (kRpStages - 1);
+            pf_stage = (gpos + i + kRpStages - 1) % kRpStages;
             if (!spread && filler && (!final_step || i + kRpStages - 1 < ncb)) fill(pf_cbi, pf_stage);
             __builtin_amdgcn_sched_barrier(0);
         };
@@ -520,7 +532,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             const bool ragged = (N & (kRpCols - 1)) != 0;
             // chunk 0: nothing to do arithmetic on yet; sweep 1 takes its reference from the first half
             {
-                const int stage = gpos & (kRpStages - 1);
+                const int stage = gpos % kRpStages;
                 sync(0, Fill::value);
                 half(I0{}, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
                 if (MODE == kRoleSum && my_role == kRoleSum) stats_reference();
@@ -529,14 +541,14 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             // chunk 1: completes chunk 0, whose window is an edge
             {
                 sync(1, Fill::value);
-                const int stage = (gpos + 1) & (kRpStages - 1);
+                const int stage = (gpos + 1) % kRpStages;
                 half(mode_c, I0{}, True{}, Fill{}, False{}, False{}, stage, 0, pf_cbi, pf_stage);
                 if (MODE == kRoleOut) ring_store_edge(0);
                 half(mode_c, I1{}, True{}, Fill{}, False{}, False{}, stage, 1, pf_cbi, pf_stage);
             }
             for (int i = 2; i < ncb - 1; ++i) {
                 sync(i, Fill::value);
-                const int stage = (gpos + i) & (kRpStages - 1);
+                const int stage = (gpos + i) % kRpStages;
                 half(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
                 half(mode_c, I1{}, True{}, Fill{}, False{}, Out{}, stage, i, pf_cbi, pf_stage);
             }
@@ -544,7 +556,7 @@ __global__ __launch_bounds__(kRpThreads, 1) void rowpipe_kernel(RunArgs a, int z
             {
                 const int i = ncb - 1;
                 sync(i, Fill::value);
-                const int stage = (gpos + i) & (kRpStages - 1);
+                const int stage = (gpos + i) % kRpStages;
                 half(mode_c, I0{}, True{}, Fill{}, False{}, Out{}, stage, i - 1, pf_cbi, pf_stage);
                 if (MODE != kRoleOut && ragged) {
                     half(mode_c, I1{}, True{}, Fill{}, True{}, False{}, stage, i, pf_cbi, pf_stage);

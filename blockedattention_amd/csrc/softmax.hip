@@ -189,7 +189,7 @@ __device__ __forceinline__ void softmax_runs(const SoftmaxArgs &a, int64_t seg0,
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (r0 + 4 * e < rows)
-                    store_run<DT == BA_BF16 ? 1 : 0, G, DT == BA_F32>(
+                    store_run<DT == BA_BF16 ? 1 : 0, G, DT == BA_F32, true>(
                         reinterpret_cast<char *>(dst + (int64_t)(r0 + 4 * e) * cols), x, e);
         }
     }
@@ -256,8 +256,8 @@ template <int DT> struct Raw8 {
         for (int i = 0; i < 4; ++i) { x[2 * i] = Io<DT>::lo(a[i]); x[2 * i + 1] = Io<DT>::hi(a[i]); }
     }
     static __device__ __forceinline__ void store(T *p, const float (&x)[8]) {
-        *reinterpret_cast<u32x4_unaligned *>(p) = u32x4{Io<DT>::pack(x[0], x[1]), Io<DT>::pack(x[2], x[3]),
-                                                        Io<DT>::pack(x[4], x[5]), Io<DT>::pack(x[6], x[7])};
+        store_result<false>(reinterpret_cast<u32x4_unaligned *>(p), u32x4{Io<DT>::pack(x[0], x[1]), Io<DT>::pack(x[2], x[3]),
+                                                                   Io<DT>::pack(x[4], x[5]), Io<DT>::pack(x[6], x[7])});
     }
 };
 template <> struct Raw8<BA_F32> {
@@ -272,8 +272,8 @@ template <> struct Raw8<BA_F32> {
         for (int i = 0; i < 4; ++i) { x[i] = a[i]; x[4 + i] = b[i]; }
     }
     static __device__ __forceinline__ void store(T *p, const float (&x)[8]) {
-        *reinterpret_cast<f32x4_unaligned *>(p) = f32x4{x[0], x[1], x[2], x[3]};
-        *reinterpret_cast<f32x4_unaligned *>(p + 4) = f32x4{x[4], x[5], x[6], x[7]};
+        store_result<false>(reinterpret_cast<f32x4_unaligned *>(p), f32x4{x[0], x[1], x[2], x[3]});
+        store_result<false>(reinterpret_cast<f32x4_unaligned *>(p + 4), f32x4{x[4], x[5], x[6], x[7]});
     }
 };
 // Forward softmax of rows first, first + stride, ... of one segment whose rows take STEPS 512-column

@@ -152,7 +152,7 @@ __device__ __forceinline__ void store_quad(void *__restrict__ out, int64_t e, co
     if (F32OUT) {
         float *o = reinterpret_cast<float *>(out) + e;
         if (valid >= 4) {
-            *reinterpret_cast<f32x4_unaligned *>(o) = v;
+            store_result<false>(reinterpret_cast<f32x4_unaligned *>(o), v);
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -161,7 +161,7 @@ __device__ __forceinline__ void store_quad(void *__restrict__ out, int64_t e, co
     } else {
         uint16_t *o = reinterpret_cast<uint16_t *>(out) + e;
         if (valid >= 4) {
-            *reinterpret_cast<u32x2_unaligned *>(o) = u32x2{Elem<DT>::pack2(v[0], v[1]), Elem<DT>::pack2(v[2], v[3])};
+            store_result<false>(reinterpret_cast<u32x2_unaligned *>(o), u32x2{Elem<DT>::pack2(v[0], v[1]), Elem<DT>::pack2(v[2], v[3])});
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -561,11 +561,11 @@ __device__ __forceinline__ void strips_exact(const Seg &s, const RunArgs &a, uns
             const int row_stride4 = 4 * N * kOutBytes;
             if (r0 + kStripRows <= M) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) store_run<DT, G, F32OUT>(dst + e * row_stride4, acc, e);
+                for (int e = 0; e < 4; ++e) store_run<DT, G, F32OUT, true>(dst + e * row_stride4, acc, e);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (r0 + 4 * e + rg < M) store_run<DT, G, F32OUT>(dst + e * row_stride4, acc, e);
+                    if (r0 + 4 * e + rg < M) store_run<DT, G, F32OUT, true>(dst + e * row_stride4, acc, e);
             }
         }
     }
