@@ -66,8 +66,9 @@ typedef uint32_t __attribute__((aligned(2))) u32_unaligned;
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef f32x2 __attribute__((aligned(4))) f32x2_unaligned;
 
-// Results are written once and not read again by the kernel that writes them.  As NON-TEMPORAL stores they do not
-// push the operands that ARE read again out of the L2, and reads no longer queue behind the write stream -- where
+// Results are written once and not read again by the kernel that writes them.  As ordinary stores they delay the
+// kernel's own reads (the operand fills of a large-segment kernel wait behind its write stream: 2500 cycles per
+// chunk against 540 with the stores compiled out); as NON-TEMPORAL stores they do so much less -- where
 // a kernel writes whole lines.  Measured per kernel, non-temporal against ordinary stores: pipelined row-block
 // kernel 1365 / 1478 us and the product alone 1000 / 1206 us (16 x 16 pairs of 1024..4096 rows), lane-run softmax
 // 12.2 / 13.4 us (256 x 8 heads); but the any-layout GEMM 2226 / 1663 us (its 8- and 16-byte pieces end in partial

@@ -58,10 +58,9 @@ constexpr int kRpRingPitch = 296;                         // 128 columns + a cop
 constexpr int kRpRingBytes = kRpWaveRows * kRpRingPitch;  // per wavefront of a set
 constexpr int kRpFlagOffset = kRpStages * kRpStageBytes + kRpSetWaves * kRpRingBytes;
 constexpr int kRpLdsBytes = kRpFlagOffset + 64;
-// Cache policy of the result stores: non-temporal.  The results are written once and never read by this kernel; as
-// ordinary stores they push the chunks of B_g, which every step reads again, out of the die's L2, and the fills then
-// wait behind the write stream (measured: the filling set waits 2500 cycles per iteration for its chunk with the
-// stores, 540 without them; 16 x 16 pairs of 1024..4096 rows and columns: 1490 us -> 1395 us with this bit).
+// Cache policy of the result stores: non-temporal.  As ordinary stores they delay the fills of B_g, which every step
+// reads again: the filling set waits 2500 cycles per iteration for its chunk with the stores, 540 without them
+// (16 x 16 pairs of 1024..4096 rows and columns: 1490 us -> 1365 us with this bit).
 constexpr int kRpStoreAux = kResultAux;
 constexpr uint32_t kRpOutOfRange = 0x80000000u;           // byte offset no segment reaches (areas are below 2^31 bytes)
 
