@@ -19,7 +19,7 @@ SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
     "ba_plan_read_into", "ba_plan_gemm_notify", "ba_plan_softmax_notify", "ba_plan_wait",
     "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax",
-    "ba_varlen_attention", "ba_gemm_softmax_static",
+    "ba_varlen_attention", "ba_gemm_softmax_static", "ba_static_read",
 )
 MAILBOX_BYTES = 320
 STATIC_MAX_SEGMENTS = 4096   # BA_STATIC_MAX_SEGMENTS
@@ -93,6 +93,8 @@ def load():
     lib.ba_varlen_attention.argtypes = [vp, ctypes.POINTER(PlanInfo), i64, i32, vp, vp, vp, vp, i64, i64, i64, i64, f32, vp]
     lib.ba_gemm_softmax_static.restype = i32
     lib.ba_gemm_softmax_static.argtypes = [i64, i32, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
+    lib.ba_static_read.restype = i32
+    lib.ba_static_read.argtypes = [vp, vp]
     _lib = lib
     return lib
 
@@ -252,6 +254,15 @@ def gemm_softmax_static(MList, NList, KList, A, B, out, H, Dm1, Dm2, Dout, scale
                                        dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
     check(st, "ba_gemm_softmax_static")
     return out
+
+
+def static_read(raise_on_bad=True):
+    """Summary of the last gemm_softmax_static call on the current stream (see ba_static_read)."""
+    info = PlanInfo()
+    st = load().ba_static_read(ctypes.byref(info), _stream())
+    if st != 0 and (raise_on_bad or st != 5):
+        check(st, "ba_static_read")
+    return info, st
 
 
 def varlen_attention(plan, Q, K, V, out, H, Dm1, Dm2, Dout, scale=1.0):

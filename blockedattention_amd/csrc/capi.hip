@@ -265,7 +265,9 @@ __attribute__((visibility("default"))) int ba_gemm_softmax_static(int64_t nseg, 
         if (mode < 0 || mode > 2 || !MList || !NList || !KList) return BA_ERR_INVALID_ARG;
         if (mode == BA_META_GIVEN && (!accum1 || !accum2 || !accumOut)) return BA_ERR_INVALID_ARG;
         if (!out || (Dm1 > 0 && !A) || (Dm2 > 0 && !B)) return BA_ERR_INVALID_ARG;
-        RunArgs args{nullptr, A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, 0, (int)nseg};
+        // (the buffer's first 256 bytes take the verdict of the call: see ba_static_read)
+        RunArgs args{static_plan_buffer(), A, B, out, H, Dm1, Dm2, Dout, scale, 0, 0, 0, (int)nseg};
+        if (!args.plan) return BA_ERR_LAUNCH;
         args.flags |= mfma_flag(args);
         if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
         return launch_onecall(dtype, args, mode, MList, NList, KList, accum1, accum2, accumOut, (hipStream_t)stream);
@@ -283,6 +285,13 @@ __attribute__((visibility("default"))) int ba_gemm_softmax_static(int64_t nseg, 
     args.flags |= mfma_flag(args);
     if (out_dtype == BA_F32) args.flags |= kFlagOutF32;
     return launch_strips(dtype, 1, args, nseg, nullptr, (hipStream_t)stream);
+}
+
+__attribute__((visibility("default"))) int ba_static_read(ba_plan_info *info, ba_stream_t stream) {
+    if (!info) return BA_ERR_INVALID_ARG;
+    void *plan = static_plan_buffer();
+    if (!plan) return BA_ERR_LAUNCH;
+    return ba_plan_read(plan, info, stream);
 }
 
 __attribute__((visibility("default"))) int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg,

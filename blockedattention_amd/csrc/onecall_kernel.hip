@@ -61,6 +61,7 @@ __global__ __launch_bounds__(kSegThreads, 2) void onecall_kernel(RunArgs a, Meta
         int64_t pre1 = 0, pre2 = 0, preO = 0, tot1 = 0, tot2 = 0, totO = 0, weight = 0;
         int64_t my_m = 0, my_n = 0, my_k = 0;
         bool any_bad = false;
+        int nbad = 0;
 #pragma unroll
         for (int q = 0; q < kRounds; ++q) {
             if (q >= m.rounds) break;
@@ -77,7 +78,8 @@ __global__ __launch_bounds__(kSegThreads, 2) void onecall_kernel(RunArgs a, Meta
                 bad = bad || mm[q] * kk[q] >= lim || nn[q] * kk[q] >= lim || mm[q] * nn[q] >= lim;
                 if (bad) { mm[q] = nn[q] = kk[q] = 0; }
             }
-            any_bad = any_bad || __ballot(bad) != 0;
+            nbad += __builtin_popcountll(__ballot(bad));
+            any_bad = nbad != 0;
             const int64_t v1 = mm[q] * kk[q], v2 = nn[q] * kk[q], vO = mm[q] * nn[q];
             const int32_t mi = (int32_t)mm[q], ni = (int32_t)nn[q];
             const int32_t strips = ni >= 1 ? (mi + kStripRows - 1) / kStripRows : 0;
@@ -125,6 +127,18 @@ __global__ __launch_bounds__(kSegThreads, 2) void onecall_kernel(RunArgs a, Meta
                         D2 == a.Dm2 && DO == a.Dout;
         if (lane == 0) {
             box[0] = o1; box[1] = o2; box[2] = oO; box[3] = my_m; box[4] = my_n; box[5] = my_k; box[6] = ok ? 1 : 0;
+        }
+        // The verdict, where the caller gave a place for it: a plan header without lists, with what the scheduler
+        // would have reported (rejected segments, or totals that do not match the call as a run error).
+        if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && lane == 0 && a.plan) {
+            PlanHeader hd = {};
+            hd.magic = kPlanMagic;
+            hd.nseg = nseg;
+            hd.cap = (int32_t)plan_cap(nseg);
+            hd.Dm1 = D1; hd.Dm2 = D2; hd.Dout = DO;
+            hd.bad_segments = nbad + ((D1 < 0 || D2 < 0 || DO < 0) ? 1 : 0) + (weight >= (int64_t(1) << 31) ? 1 : 0);
+            hd.run_errors = hd.bad_segments == 0 && !ok ? 1 : 0;
+            *reinterpret_cast<PlanHeader *>(a.plan) = hd;
         }
     }
     __syncthreads();

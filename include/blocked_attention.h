@@ -241,8 +241,8 @@ int ba_varlen_attention(void *plan, const ba_plan_info *info, int64_t nseg, int 
  * Nothing is allocated and nothing is read back: the kernels take their work
  * lists from the plan on the device, exactly as ba_gemm_softmax does with
  * info == NULL, and give the same results.  Metadata the scheduler rejects
- * leaves `out` unwritten (there is no summary to report it through), so check
- * new metadata once with ba_plan_gemm + ba_plan_read.
+ * leaves `out` unwritten; ba_static_read (below) tells, at the price of a
+ * synchronisation.
  * The FIRST call on a device looks up the buffer's address and sets kernel
  * attributes (host-side calls that do not belong in a stream capture): make
  * one call per device outside any capture, with any small batch, before the
@@ -263,6 +263,13 @@ int ba_gemm_softmax_static(int64_t nseg, int mode, int64_t *MList, int64_t *NLis
                            int64_t *accum1, int64_t *accum2, int64_t *accumOut, int dtype, const void *A,
                            const void *B, void *out, int out_dtype, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
                            float scale, ba_stream_t stream);
+
+/* ba_plan_read on the buffer of ba_gemm_softmax_static (current device): the verdict of the LAST call of that entry
+ * point on `stream` -- BA_ERR_BAD_METADATA with bad_segments / run_errors set when that call's metadata was
+ * rejected or its totals did not match the sizes passed, in which case it wrote nothing.  Blocks like ba_plan_read
+ * (so not for use under stream capture); after a single-launch call only nseg, Dm1, Dm2, Dout, bad_segments and
+ * run_errors of the summary are meaningful.  No counterpart in the reference. */
+int ba_static_read(ba_plan_info *host_info, ba_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -80,12 +80,18 @@ def test_rejected_metadata_leaves_the_output_alone(dev):
     capi.gemm_softmax_static(dev_i64(bad_M, dev), dev_i64(N, dev), dev_i64(K, dev), Ad, Bd, out, 1, d1, d2, do, 1.0)
     torch.cuda.synchronize()
     assert torch.isnan(out).all(), "a negative size must stop the whole call"
+    info, st = capi.static_read(raise_on_bad=False)
+    assert st == 5 and info.bad_segments == 1 and info.nseg == 3, (st, info.bad_segments, info.nseg)
     capi.gemm_softmax_static(dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev), Ad, Bd, out, 1, d1, d2, do + 8, 1.0)
     torch.cuda.synchronize()
     assert torch.isnan(out).all(), "totals that do not match the tensors' sizes must stop the whole call"
+    info, st = capi.static_read(raise_on_bad=False)
+    assert st == 5 and info.bad_segments == 0 and info.run_errors >= 1, (st, info.bad_segments, info.run_errors)
     capi.gemm_softmax_static(dev_i64(M, dev), dev_i64(N, dev), dev_i64(K, dev), Ad, Bd, out, 1, d1, d2, do, 1.0)
     torch.cuda.synchronize()
     assert_probs_close(out, oracle.per_segment_torch(A, B, M, N, K, 1.0), "after the rejected calls")
+    info, st = capi.static_read()
+    assert st == 0 and info.bad_segments == 0 and info.run_errors == 0 and info.Dout == do
 
 
 def test_prefix_sums_given_by_the_caller_with_gaps(dev):
@@ -218,6 +224,8 @@ def test_given_prefix_sums_that_overlap_are_rejected(dev):
                              1.0, dev_i64(a1, dev), dev_i64(a2, dev), dev_i64(ao, dev), mode=capi.META_GIVEN)
     torch.cuda.synchronize()
     assert torch.isnan(out).all()
+    info, st = capi.static_read(raise_on_bad=False)
+    assert st == 5 and info.bad_segments >= 1
 
 
 def test_many_heads_up_to_the_pair_limit_and_beyond(dev):
