@@ -18,7 +18,8 @@ enum RunFlags : int {
     kFlagQuiet = 64,       // an earlier launch of the same call reports a plan that does not match
     kFlagSmallToo = 128,   // strip kernel, 64 KiB launch: the slots from both_split on walk the main launch's list
     kFlagHeadFast = 256,   // strip kernel: grid (head, slot, z) instead of (slot, head, z)
-    kFlagPipeToo = 512     // tile kernel: the pipelined row-block kernel runs in the same call and takes its segments
+    kFlagPipeToo = 512,    // tile kernel: the pipelined row-block kernel runs in the same call and takes its segments
+    kFlagRingToo = 1024    // any-layout GEMM: the ring kernel runs in the same call and takes its segments
 };
 
 struct RunArgs {

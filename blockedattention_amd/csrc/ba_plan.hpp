@@ -106,7 +106,9 @@ struct PlanHeader {
     int32_t mini_count;      // total of kPfxMini
     int32_t pipe_count;      // total of kPfxPipe
     int32_t pipe_groups;     // bumped by every workgroup of the pipelined row-block kernel that found work in this plan
-    int32_t pad_[16];
+    int32_t min_N, min_K;    // smallest N and K over the segments that have rows and columns (0: there is none)
+    int32_t ring_groups;     // bumped by every workgroup of the any-layout GEMM that wrote its rows through the LDS ring
+    int32_t pad_[13];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 

@@ -126,6 +126,8 @@ static int info_from_header(const PlanHeader &h, ba_plan_info *info) {
     info->list_mini = h.mini_count;
     info->list_pipe = h.pipe_count;
     info->pipe_groups = h.pipe_groups;
+    info->min_N = h.min_N; info->min_K = h.min_K;
+    info->ring_groups = h.ring_groups;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 

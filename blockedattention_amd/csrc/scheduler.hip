@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     constexpr int kNumScan = kNumPrefix + (kBucketed ? kSmallBuckets / 2 : 0);   // scanned words
     __shared__ int64_t sScan64[16 * 3];
     __shared__ int32_t sScan32[16 * kNumScan];
-    __shared__ int32_t sRed[kSchedWaves][6];
+    __shared__ int32_t sRed[kSchedWaves][8];
     __shared__ int64_t sWeight[kSchedWaves];
 
     const int tid = threadIdx.x;
@@ -133,6 +133,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     int32_t base32[kNumPrefix] = {};
     int32_t maxM = 0, maxN = 0, maxK = 0, nbad = 0;
     int32_t maxSmallN = 0, maxSmallM = 0;       // widest / tallest segment of the strip kernel's main launch
+    int32_t maxInvN = 0, maxInvK = 0;           // INT32_MAX - the smallest N and K of the segments that have rows and columns
     // Every scanned count of a segment is at most max(rows, strips x chunks): while the sum of these weights stays
     // below 2^31, none of the int32 scans can overflow; a batch beyond that is rejected as a whole.
     int64_t weight = 0;
@@ -300,6 +301,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         }
         maxM = max(maxM, mi); maxN = max(maxN, ni); maxK = max(maxK, ki); nbad += bad ? 1 : 0;
         if (cls == kListSmall) { maxSmallN = max(maxSmallN, ni); maxSmallM = max(maxSmallM, mi); }
+        if (mi >= 1 && ni >= 1) { maxInvN = max(maxInvN, INT32_MAX - ni); maxInvK = max(maxInvK, INT32_MAX - ki); }
 #pragma unroll
         for (int q = 0; q < kNumPrefix; ++q) base32[q] += t32[q];
         if (!offsets_given) {
@@ -314,11 +316,12 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
     // wavefront, then thread 0 folds the 16 partial results.
     maxM = wave_max_nonneg(maxM); maxN = wave_max_nonneg(maxN); maxK = wave_max_nonneg(maxK);
     maxSmallN = wave_max_nonneg(maxSmallN); maxSmallM = wave_max_nonneg(maxSmallM);
+    maxInvN = wave_max_nonneg(maxInvN); maxInvK = wave_max_nonneg(maxInvK);
     nbad = __builtin_amdgcn_readlane(wave_inclusive_scan(nbad), 63);
 #pragma unroll
     for (int msk = 32; msk >= 1; msk >>= 1) weight += __shfl_xor(weight, msk);
     if (lane == 0) sWeight[wave] = weight;
-    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; sRed[wave][4] = maxSmallN; sRed[wave][5] = maxSmallM; }
+    if (lane == 0) { sRed[wave][0] = maxM; sRed[wave][1] = maxN; sRed[wave][2] = maxK; sRed[wave][3] = nbad; sRed[wave][4] = maxSmallN; sRed[wave][5] = maxSmallM; sRed[wave][6] = maxInvN; sRed[wave][7] = maxInvK; }
     __syncthreads();
 
     if (tid == 0) {
@@ -333,12 +336,12 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
             if (a.a2) a.a2[nseg] = D2;
             if (a.aO) a.aO[nseg] = DO;
         }
-        int32_t rM = 0, rN = 0, rK = 0, rBad = 0, rSN = 0, rSM = 0;
+        int32_t rM = 0, rN = 0, rK = 0, rBad = 0, rSN = 0, rSM = 0, rInvN = 0, rInvK = 0;
         int64_t total_weight = 0;
         for (int w = 0; w < kSchedWaves; ++w) {
             rM = max(rM, sRed[w][0]); rN = max(rN, sRed[w][1]); rK = max(rK, sRed[w][2]); rBad += sRed[w][3];
             total_weight += sWeight[w];
-            rSN = max(rSN, sRed[w][4]); rSM = max(rSM, sRed[w][5]);
+            rSN = max(rSN, sRed[w][4]); rSM = max(rSM, sRed[w][5]); rInvN = max(rInvN, sRed[w][6]); rInvK = max(rInvK, sRed[w][7]);
         }
         PlanHeader *h = pv.hdr;
         h->magic = kPlanMagic;
@@ -357,6 +360,9 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->mini_count = base32[kPfxMini];
         h->pipe_count = base32[kPfxPipe];
         h->pipe_groups = 0;
+        h->min_N = rInvN ? INT32_MAX - rInvN : 0;
+        h->min_K = rInvK ? INT32_MAX - rInvK : 0;
+        h->ring_groups = 0;
         plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
         plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
         if (a.mailbox) {

@@ -90,6 +90,11 @@ typedef struct ba_plan_info {
      * (K <= 128), and how many workgroups of that kernel have found work in this plan since it was built */
     int32_t list_pipe;
     int32_t pipe_groups;
+    /* smallest N and K over the segments that have rows and columns (0: none has), and how many workgroups of
+     * the GEMM for transposed layouts have written their rows as whole lines (128 x 128 build, K <= 128,
+     * N >= 128) since the plan was built */
+    int32_t min_N, min_K;
+    int32_t ring_groups;
 } ba_plan_info;
 
 const char *ba_status_string(int status);

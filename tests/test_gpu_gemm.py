@@ -77,6 +77,32 @@ def test_transposed_layouts(dev, dtype, t1, t2):
     assert_scores_close(out, torch.from_numpy(ref), f"transpose {t1} {t2}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t1,t2", [(True, False), (False, True), (True, True)])
+def test_transposed_layouts_of_tall_segments(dev, dtype, t1, t2):
+    # averages of four and more 64-row blocks per segment: the 128 x 128 build, whose segments with K <= 128 and
+    # N >= 128 write whole lines through a ring (odd N: every row at another phase; N at and around the 64-column
+    # chunk and 128-column block boundaries; rows that end inside a block); K = 136 and N = 100 take the other path
+    M = [300, 257, 512, 129, 640, 384, 1, 260, 200]; N = [128, 129, 191, 193, 255, 257, 300, 1000, 100]
+    K = [128, 64, 72, 8, 100, 40, 128, 136, 64]; H = 2
+    A, B = random_operands(M, N, K, H, dtype, seed=13)
+    plan = make_plan(dev, M, N, K)
+    assert plan.info.att_blocks64 >= 4 * len(M)
+    ref = torch.from_numpy(oracle.varlen_gemm(A.float().numpy(), B.float().numpy(), M, N, K, t1, t2, f64acc=True))
+    i = plan.info
+    for shift in (0, 1, 3):                                    # the result's base pointer at several 2-byte phases
+        flat = torch.full((H * i.Dout + 8,), float("nan"), dtype=dtype, device=dev)
+        out = flat[shift:shift + H * i.Dout].view(H, i.Dout)
+        capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, H, i.Dm1, i.Dm2, i.Dout, t1, t2)
+        assert_scores_close(out, ref, f"transpose {t1} {t2} shift {shift}")
+        assert torch.isnan(flat[:shift]).all() and torch.isnan(flat[shift + H * i.Dout:]).all(), "wrote outside the result"
+    # the plan counts the workgroups that went through the ring: 128-row rounds of the seven segments with
+    # K <= 128 and N >= 128, per head and call
+    ring_rounds = sum(-(-m // 128) for m, n, k in zip(M, N, K) if k <= 128 and n >= 128)
+    assert (plan.info.min_N, plan.info.min_K) == (100, 8)
+    assert plan.read().ring_groups == 3 * H * ring_rounds
+
+
 def test_ragged_edges_and_degenerate_segments(dev):
     # rows/cols not multiples of 16, N across the 256-column chunk boundary, K % 32 in {8,16,24},
     # K = 0 (zeros), M = 0 and N = 0 (no work), odd N (unaligned row starts in the output).
