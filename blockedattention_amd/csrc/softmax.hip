@@ -335,6 +335,75 @@ __device__ __forceinline__ void softmax_rows_forward(const typename Io<DT>::T *s
     }
 }
 
+// Backward of rows first, first + stride, ... with the row's y and dy in registers (as they were loaded: 16-bit types
+// stay packed), so that both are read from memory ONCE: dx = scale * (dy - sum(y * dy)) * y needs the row's sum before
+// its first result.  The same runs, weights and re-stored overlap as in the forward above; the next row's loads are
+// issued before the arithmetic of the current one, whose stores come after all of its loads (dst may alias y or dy).
+template <int DT, int STEPS>
+__device__ __forceinline__ void softmax_rows_backward(const typename Io<DT>::T *ysrc, const typename Io<DT>::T *gsrc,
+                                                      typename Io<DT>::T *dst, int rows, int cols, int first, int stride,
+                                                      float scale) {
+    const int lane = lane_id();
+    int at[STEPS];
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) at[k] = min(512 * k + 8 * lane, cols - 8);
+    const int own = 512 * (STEPS - 1) + 8 * lane - at[STEPS - 1];
+    float w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = (i >= own && own < 8) ? 1.f : 0.f;
+    // up to 2048 columns two rows fit the registers of a wavefront at four wavefronts per SIMD; wider rows are loaded
+    // when their turn comes, and the other wavefronts of the SIMD cover the wait
+    constexpr bool kAhead = STEPS * (DT == BA_F32 ? 2 : 1) <= 4;
+    Raw8<DT> ry[STEPS], rg[STEPS];
+    if (kAhead && first < rows) {
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) {
+            ry[k].load(ysrc + (int64_t)first * cols + at[k]);
+            rg[k].load(gsrc + (int64_t)first * cols + at[k]);
+        }
+    }
+    for (int r = first; r < rows; r += stride) {
+        Raw8<DT> cy[STEPS], cg[STEPS];
+        if constexpr (kAhead) {
+#pragma unroll
+            for (int k = 0; k < STEPS; ++k) { cy[k] = ry[k]; cg[k] = rg[k]; }
+            if (r + stride < rows) {
+#pragma unroll
+                for (int k = 0; k < STEPS; ++k) {
+                    ry[k].load(ysrc + (int64_t)(r + stride) * cols + at[k]);
+                    rg[k].load(gsrc + (int64_t)(r + stride) * cols + at[k]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < STEPS; ++k) {
+                cy[k].load(ysrc + (int64_t)r * cols + at[k]);
+                cg[k].load(gsrc + (int64_t)r * cols + at[k]);
+            }
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) {
+            float yv[8], gv[8];
+            cy[k].unpack(yv);
+            cg[k].unpack(gv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot = k < STEPS - 1 ? fmaf(yv[i], gv[i], dot) : fmaf(yv[i] * gv[i], w[i], dot);
+        }
+        dot = wave_sum(dot);
+        typename Io<DT>::T *dx = dst + (int64_t)r * cols;
+#pragma unroll
+        for (int k = 0; k < STEPS; ++k) {
+            float yv[8], gv[8], dv[8];
+            cy[k].unpack(yv);
+            cg[k].unpack(gv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dv[i] = scale * (gv[i] - dot) * yv[i];
+            Raw8<DT>::store(dx + at[k], dv);
+        }
+    }
+}
+
 template <int DT, bool BACKWARD, int MAXG>
 __global__ __launch_bounds__(kSoftmaxThreads, MAXG <= 8 ? 3 : 1) void softmax_runs_kernel(SoftmaxArgs a) {
     if (a.head_fast) softmax_runs_body<DT, BACKWARD, MAXG>(a, blockIdx.y, blockIdx.x, blockIdx.z, gridDim.z);
@@ -382,7 +451,23 @@ __device__ __forceinline__ void softmax_rows_body(const SoftmaxArgs &a, uint64_t
 #undef BA_ROWS
         return;
     }
-    // Rows wider than the register path holds, and the backward: the row is streamed in 512-column steps,
+    if (BACKWARD && steps <= (DT == BA_F32 ? kRowSteps / 2 : kRowSteps)) {
+#define BA_ROWS(S_) case S_: softmax_rows_backward<DT, S_>(src, aux, dst, rows, cols, first, stride, a.scale); break;
+        switch (steps) {
+            BA_ROWS(1) BA_ROWS(2) BA_ROWS(3) BA_ROWS(4)
+            default:
+                if constexpr (DT != BA_F32) {
+                    switch (steps) {
+                        BA_ROWS(5) BA_ROWS(6) BA_ROWS(7) BA_ROWS(8)
+                        default: break;
+                    }
+                }
+                break;
+        }
+#undef BA_ROWS
+        return;
+    }
+    // Rows wider than the register path holds (forward and backward): the row is streamed in 512-column steps,
     // four steps of loads in flight, once per pass.  A lane reads the run of eight elements that starts
     // at its column, or the run ENDING at the row's end when that would pass it; `own` is the number of
     // leading elements of the run that belong to the lanes before (8 or more: none are this lane's).

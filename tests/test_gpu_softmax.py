@@ -113,3 +113,28 @@ def test_backward_wide_ragged_rows_and_in_place(dev, dtype):
     buf = dy.to(dev).clone()                                   # dx written over dy
     capi.blocked_softmax_backward(plan, y, buf, buf, 2, y.shape[1], 1.0)
     assert torch.equal(buf, dx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_backward_rows_held_in_registers(dev, dtype):
+    # one row length per count of 512-column steps (1..8: both inputs of a row are read once and kept in registers;
+    # fp32 up to 2048 columns, the wider rows streamed twice), odd lengths, and without the host summary, so that a
+    # wavefront takes several rows one after the other (the next row's loads under the current row's arithmetic)
+    rows = [37] * 8 + [5]
+    cols = [301, 777, 1283, 2048, 2049, 2901, 3583, 4096, 4100]
+    H = 2
+    src, y, plan = run_softmax(dev, rows, cols, H, dtype, scale=0.7, seed=21)
+    g = torch.Generator().manual_seed(22)
+    dy = torch.randn(y.shape, generator=g).to(dtype)
+    ref = oracle.blocked_softmax_backward(y.float().cpu().numpy(), dy.float().numpy(), rows, cols, 0.7)
+    tol = {torch.float16: 2e-3, torch.bfloat16: 2e-2, torch.float32: 1e-6}[dtype]
+    for with_summary in (True, False):
+        if not with_summary:
+            plan.info = None
+        dx = torch.full_like(y, float("nan"))
+        capi.blocked_softmax_backward(plan, y, dy.to(dev), dx, H, y.shape[1], 0.7)
+        assert np.abs(dx.float().cpu().numpy() - ref).max() <= tol, f"summary {with_summary}"
+        buf = y.clone()                                        # dx written over y
+        capi.blocked_softmax_backward(plan, buf, dy.to(dev), buf, H, y.shape[1], 0.7)
+        assert torch.equal(buf, dx)
+
