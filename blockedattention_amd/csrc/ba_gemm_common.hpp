@@ -162,6 +162,34 @@ __device__ __forceinline__ void store_run(char *dst, const f32x4 (&acc)[G], int 
     }
 }
 
+// The same through a buffer descriptor: `off` is a byte offset inside the descriptor's range, or any value outside
+// it for a lane that has nothing to store (the hardware drops the store): no branch around the stores, so a loop that
+// loads at its top and stores at its bottom stays one block of straight-line code and the wait in front of the first
+// use of what it loaded counts the stores as still in flight instead of waiting for them.
+template <int DT, int G, bool F32OUT>
+__device__ __forceinline__ void store_run_buf(__amdgpu_buffer_rsrc_t res, uint32_t off, const f32x4 (&acc)[G], int e) {
+    if constexpr (!F32OUT) {
+        uint32_t w[G / 2];
+#pragma unroll
+        for (int k = 0; k < G / 2; ++k) w[k] = Elem<DT>::pack2(acc[2 * k][e], acc[2 * k + 1][e]);
+#pragma unroll
+        for (int k = 0; k + 4 <= G / 2; k += 4)
+            __builtin_amdgcn_raw_buffer_store_b128(u32x4{w[k], w[k + 1], w[k + 2], w[k + 3]}, res, off + 4 * k, 0, kResultAux);
+        constexpr int kDone = (G / 2) & ~3;
+        if constexpr (((G / 2) & 2) != 0)
+            __builtin_amdgcn_raw_buffer_store_b64(u32x2{w[kDone], w[kDone + 1]}, res, off + 4 * kDone, 0, kResultAux);
+        if constexpr (((G / 2) & 1) != 0) __builtin_amdgcn_raw_buffer_store_b32(w[G / 2 - 1], res, off + 4 * (G / 2 - 1), 0, kResultAux);
+    } else {
+#pragma unroll
+        for (int k = 0; k + 4 <= G; k += 4)
+            __builtin_amdgcn_raw_buffer_store_b128(
+                __builtin_bit_cast(u32x4, f32x4{acc[k][e], acc[k + 1][e], acc[k + 2][e], acc[k + 3][e]}), res, off + 4 * k, 0, kResultAux);
+        if constexpr ((G & 2) != 0)
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, f32x2{acc[G - 2][e], acc[G - 1][e]}), res,
+                                                  off + 4 * (G - 2), 0, kResultAux);
+    }
+}
+
 __device__ __forceinline__ Seg load_seg(const PlanRO &pv, int g, int64_t h, const RunArgs &a) {
     const SegRec r = load_rec(pv.recs, g);   // scalar loads
     Seg s;
