@@ -19,7 +19,7 @@ SYMBOLS = (
     "ba_status_string", "ba_abi_version", "ba_plan_bytes", "ba_plan_gemm", "ba_plan_softmax", "ba_plan_read",
     "ba_plan_read_into", "ba_plan_gemm_notify", "ba_plan_softmax_notify", "ba_plan_wait",
     "ba_varlen_gemm", "ba_blocked_softmax", "ba_blocked_softmax_backward", "ba_gemm_softmax",
-    "ba_varlen_attention", "ba_gemm_softmax_static", "ba_static_read",
+    "ba_varlen_attention", "ba_gemm_softmax_static", "ba_static_read", "ba_varlen_gemm_two",
 )
 MAILBOX_BYTES = 320
 STATIC_MAX_SEGMENTS = 4096   # BA_STATIC_MAX_SEGMENTS
@@ -95,6 +95,9 @@ def load():
     lib.ba_gemm_softmax_static.argtypes = [i64, i32, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i64, i64, i64, i64, f32, vp]
     lib.ba_static_read.restype = i32
     lib.ba_static_read.argtypes = [vp, vp]
+    lib.ba_varlen_gemm_two.restype = i32
+    lib.ba_varlen_gemm_two.argtypes = [i32, i64, vp, ctypes.POINTER(PlanInfo), vp, vp, vp, i64, i64, i64,
+                                       vp, ctypes.POINTER(PlanInfo), vp, vp, vp, i64, i64, i64, vp]
     _lib = lib
     return lib
 
@@ -254,6 +257,16 @@ def gemm_softmax_static(MList, NList, KList, A, B, out, H, Dm1, Dm2, Dout, scale
                                        dtype_code(out.dtype), H, Dm1, Dm2, Dout, float(scale), _stream())
     check(st, "ba_gemm_softmax_static")
     return out
+
+
+def varlen_gemm_two(plan_a, A_a, B_a, out_a, dims_a, plan_b, A_b, B_b, out_b, dims_b, H):
+    """Both products as one launch (see ba_varlen_gemm_two); False where the library wants two calls instead."""
+    st = load().ba_varlen_gemm_two(dtype_code(A_a.dtype), H, plan_a.ptr, plan_a._hint(), _ptr(A_a), _ptr(B_a), _ptr(out_a), *dims_a,
+                                   plan_b.ptr, plan_b._hint(), _ptr(A_b), _ptr(B_b), _ptr(out_b), *dims_b, _stream())
+    if st == 3:
+        return False
+    check(st, "ba_varlen_gemm_two")
+    return True
 
 
 def static_read(raise_on_bad=True):

@@ -76,6 +76,10 @@ constexpr int64_t kOneCallMaxElements = int64_t(1) << 24;
 int launch_onecall(int dtype, const RunArgs &args, int mode, const int64_t *M, const int64_t *N, const int64_t *K,
                    int64_t *a1, int64_t *a2, int64_t *aO, hipStream_t stream);
 int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
+// Two such calls with the layouts of the backward pass (a: B operand k-major; b: both operands k-major) as ONE launch
+// where both take the 64 x 64 build; BA_ERR_UNSUPPORTED (nothing launched) otherwise.
+int launch_gemm_any16_two(int dtype, const RunArgs &a, const ba_plan_info *info_a, const RunArgs &b, const ba_plan_info *info_b,
+                          hipStream_t stream);
 // fp32, fp64 and the integer types (gemm_generic.hip); dtype: ba_dtype
 int launch_gemm_generic(int dtype, const RunArgs &args, int64_t nseg, const ba_plan_info *info, hipStream_t stream);
 int launch_softmax(int dtype, void *plan, int64_t nseg, const void *src, void *dst, int64_t H, int64_t Dsrc,

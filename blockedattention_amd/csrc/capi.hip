@@ -213,6 +213,25 @@ __attribute__((visibility("default"))) int ba_varlen_gemm(void *plan, const ba_p
     return launch_strips(dtype, 0, args, nseg, info, (hipStream_t)stream);
 }
 
+// ba_varlen_gemm twice -- (plan_a: out_a = A_a B_a^T with B_a stored K x N) and (plan_b: out_b = A_b B_b^T with both
+// operands stored k-major) -- as one launch, where that is possible; BA_ERR_UNSUPPORTED, with nothing launched, where
+// it is not (the caller then makes the two calls).
+__attribute__((visibility("default"))) int ba_varlen_gemm_two(int dtype, int64_t H, void *plan_a, const ba_plan_info *info_a,
+                                                              const void *A_a, const void *B_a, void *out_a, int64_t Dm1_a,
+                                                              int64_t Dm2_a, int64_t Dout_a, void *plan_b,
+                                                              const ba_plan_info *info_b, const void *A_b, const void *B_b,
+                                                              void *out_b, int64_t Dm1_b, int64_t Dm2_b, int64_t Dout_b,
+                                                              ba_stream_t stream) {
+    if (!plan_a || !plan_b || !info_a || !info_b) return BA_ERR_UNSUPPORTED;
+    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
+    if (bad_sizes(H, Dm1_a, Dm2_a, Dout_a) || bad_sizes(H, Dm1_b, Dm2_b, Dout_b)) return BA_ERR_INVALID_ARG;
+    if (H == 0 || Dout_a == 0 || Dout_b == 0 || info_a->nseg <= 0 || info_b->nseg <= 0) return BA_ERR_UNSUPPORTED;
+    if (!out_a || !out_b || !A_a || !B_a || !A_b || !B_b) return BA_ERR_UNSUPPORTED;
+    RunArgs a{plan_a, A_a, B_a, out_a, H, Dm1_a, Dm2_a, Dout_a, 1.0f, kFlagTranspose2, 0, 0, (int)info_a->nseg};
+    RunArgs b{plan_b, A_b, B_b, out_b, H, Dm1_b, Dm2_b, Dout_b, 1.0f, kFlagTranspose1 | kFlagTranspose2, 0, 0, (int)info_b->nseg};
+    return launch_gemm_any16_two(dtype, a, info_a, b, info_b, (hipStream_t)stream);
+}
+
 __attribute__((visibility("default"))) int ba_blocked_softmax(void *plan, const ba_plan_info *info, int64_t nseg,
                                                               int dtype,
                                                               const void *src, void *dst, int64_t H, int64_t Dsrc,

@@ -565,16 +565,20 @@ __device__ __forceinline__ void any16_stream_round(__amdgpu_buffer_rsrc_t resX, 
 // skips those when kFlagRingToo says that the ring kernel runs in the same call.  Two kernels, not one that chooses
 // per segment: either round wants all 256 registers, and neither as a function called from the other's kernel nor
 // inlined beside it did they keep out of each other's way (spills in the streaming loop, saves around every call).
+// block_x: the workgroup's index in the flat grid of a launch with the totals on the host (ride_slots = 1).
 template <int DT, int RT, int CG, bool T1, bool T2, bool RING>
-__global__ __launch_bounds__(kAnyThreads, RT * CG >= 4 ? 2 : 4) void gemm_any16_kernel(RunArgs a) {
+__device__ __forceinline__ void any16_workgroup(const RunArgs &a, unsigned block_x, unsigned char *any_lds) {
     static_assert(!RING || (RT == 2 && CG == 2), "the ring belongs to the 128 x 128 build");
-    extern __shared__ __attribute__((aligned(16))) unsigned char any_lds[];
     constexpr int kRows = kAnyTile * RT, kCols = kAnyTile * CG;
     const ConstHdr hdr = (ConstHdr)(uintptr_t)a.plan;
     const int nseg = hdr->nseg;
     const int64_t per_head = RT == 2 ? hdr->att_blocks128 : hdr->att_blocks64;   // row rounds per head
     if (!header_ok(a)) {
-        if (!(a.flags & kFlagQuiet)) report_mismatch(a);
+        if (!(a.flags & kFlagQuiet)) {
+            if (!a.ride_slots) report_mismatch(a);
+            else if (block_x == 0 && threadIdx.x == 0)       // (the first workgroup of THIS product, wherever it lies in the grid)
+                atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+        }
         return;
     }
     // Two grids.  With the batch's totals on the host (ride_slots = 1): one workgroup per existing
@@ -591,7 +595,7 @@ __global__ __launch_bounds__(kAnyThreads, RT * CG >= 4 ? 2 : 4) void gemm_any16_
         // (head slowest, then segment, then row round) are dealt to the dies in blocks of kAnyDieBlock consecutive
         // items: the workgroups a die runs together are then neighbouring row rounds of one segment and head, which
         // read the same Y, so Y comes out of that die's L2 instead of being streamed from memory once per round.
-        const int64_t u = blockIdx.x;
+        const int64_t u = block_x;
         const int64_t slot = u / kDies;
         const int64_t v = ((slot / kAnyDieBlock) * kDies + u % kDies) * kAnyDieBlock + slot % kAnyDieBlock;
         if (v >= per_head * a.H) return;
@@ -626,6 +630,23 @@ __global__ __launch_bounds__(kAnyThreads, RT * CG >= 4 ? 2 : 4) void gemm_any16_
         // the next round's first chunks may take either buffer, and go where the rings are
         if (round + round_step < rounds) lds_barrier();
     }
+}
+
+template <int DT, int RT, int CG, bool T1, bool T2, bool RING>
+__global__ __launch_bounds__(kAnyThreads, RT * CG >= 4 ? 2 : 4) void gemm_any16_kernel(RunArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char any_lds[];
+    any16_workgroup<DT, RT, CG, T1, T2, RING>(a, blockIdx.x, any_lds);
+}
+
+// Two products in one launch (64 x 64 build, totals on the host): the first `split` workgroups are those of a launch
+// over `a`, the rest those of a launch over `b`.  For the two products of the backward pass of a batch of short
+// segments, dA = dS B (second operand k-major) and dB = dS^T A (both k-major): each alone is a few rounds of
+// workgroups that live for one or two steps, and two launches pay the ramps at both ends twice.
+template <int DT>
+__global__ __launch_bounds__(kAnyThreads, 4) void gemm_any16_two_kernel(RunArgs a, RunArgs b, unsigned split) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char any_lds[];
+    if (blockIdx.x < split) any16_workgroup<DT, 1, 1, false, true, false>(a, blockIdx.x, any_lds);
+    else any16_workgroup<DT, 1, 1, true, true, false>(b, blockIdx.x - split, any_lds);
 }
 
 template <int DT, int RT, int CG, bool T1, bool T2, bool RING>
@@ -693,6 +714,37 @@ int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_pla
             else launch_any<1, 1, 1>(run, grid, stream);
         }
     }
+    return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+}
+
+// The two-product launch above, if both calls would take the 64 x 64 build with the plan's totals on the host and
+// have the layouts of the backward pass (a: second operand k-major; b: both); BA_ERR_UNSUPPORTED otherwise, and the
+// caller makes two calls of launch_gemm_any16.
+int launch_gemm_any16_two(int dtype, const RunArgs &a, const ba_plan_info *info_a, const RunArgs &b, const ba_plan_info *info_b,
+                          hipStream_t stream) {
+    if (dtype != BA_F16 && dtype != BA_BF16) return BA_ERR_UNSUPPORTED;
+    if (!info_a || !info_b || a.H != b.H || a.H > 65535) return BA_ERR_UNSUPPORTED;
+    static const int tile_env = [] { const char *e = getenv("BLOCKEDATTN_ANY_TILE"); return e ? atoi(e) : 0; }();
+    auto big = [&](const ba_plan_info *i) { return tile_env ? tile_env == 128 : (int64_t)i->att_blocks64 >= 4 * (int64_t)i->nseg; };
+    if (big(info_a) || big(info_b)) return BA_ERR_UNSUPPORTED;
+    const int layout = kFlagTranspose1 | kFlagTranspose2;
+    if ((a.flags & layout) != kFlagTranspose2 || (b.flags & layout) != layout) return BA_ERR_UNSUPPORTED;
+    const int64_t unit = (int64_t)kDies * kAnyDieBlock;
+    const int64_t items_a = (int64_t)info_a->att_blocks64 * a.H, items_b = (int64_t)info_b->att_blocks64 * b.H;
+    if (items_a <= 0 || items_b <= 0) return BA_ERR_UNSUPPORTED;
+    const int64_t grid_a = (items_a + unit - 1) / unit * unit, grid_b = (items_b + unit - 1) / unit * unit;
+    if (grid_a + grid_b >= (int64_t(1) << 31) - 1024) return BA_ERR_UNSUPPORTED;
+    RunArgs ra = a, rb = b;
+    ra.ride_slots = rb.ride_slots = 1;
+    ra.nseg = (int)info_a->nseg;
+    rb.nseg = (int)info_b->nseg;
+    constexpr int kLds = 2 * (AnyBuf<kAnyTile>::bytes + AnyBuf<kAnyTile>::bytes);
+    if (dtype == BA_F16)
+        hipLaunchKernelGGL((gemm_any16_two_kernel<0>), dim3((unsigned)(grid_a + grid_b)), dim3(kAnyThreads), kLds, stream, ra, rb,
+                           (unsigned)grid_a);
+    else
+        hipLaunchKernelGGL((gemm_any16_two_kernel<1>), dim3((unsigned)(grid_a + grid_b)), dim3(kAnyThreads), kLds, stream, ra, rb,
+                           (unsigned)grid_a);
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
 }
 

@@ -354,9 +354,27 @@ public:
         // kernels for any layout and reduction length (two launches, like the reference)
         Schedule fwd = schedule_gemm(grad, a1, a2, aO, M, N, K);          // the forward's, from the cache
         Schedule &s1 = derived_schedule(fwd, &Derived::grad1, grad, aO, a2, a1, M, K, N);
-        g1 = gemm_launch(grad, mat2, s1, false, !t2);
         Schedule &s2 = derived_schedule(fwd, &Derived::grad2, grad, aO, a1, a2, N, K, M);
-        g2 = gemm_launch(grad, mat1, s2, true, !t1);
+        // batches of short segments: both products as ONE launch where the library offers it (layouts of the
+        // untransposed forward), else one call each
+        bool done = false;
+        if (!t1 && !t2 && grad.dim() >= 1 && grad.size(-1) == s1.info.Dm1 && mat2.size(-1) == s1.info.Dm2 &&
+            grad.size(-1) == s2.info.Dm1 && mat1.size(-1) == s2.info.Dm2 && leading(mat1) == leading(grad) &&
+            leading(mat2) == leading(grad) && (grad.scalar_type() == at::kHalf || grad.scalar_type() == at::kBFloat16)) {
+            const int64_t H = leading(grad);
+            g1 = at::empty({H, s1.info.Dout}, grad.options());
+            g2 = at::empty({H, s2.info.Dout}, grad.options());
+            const int st = ba_varlen_gemm_two(dtype_code(grad, "sparseBlockedGEMM backward"), H, s1.plan.data_ptr(), &s1.info,
+                                              grad.data_ptr(), mat2.data_ptr(), g1.data_ptr(), s1.info.Dm1, s1.info.Dm2,
+                                              s1.info.Dout, s2.plan.data_ptr(), &s2.info, grad.data_ptr(), mat1.data_ptr(),
+                                              g2.data_ptr(), s2.info.Dm1, s2.info.Dm2, s2.info.Dout, current_stream(grad));
+            if (st == BA_OK) done = true;
+            else if (st != BA_ERR_UNSUPPORTED) check_status(st, "ba_varlen_gemm_two");
+        }
+        if (!done) {
+            g1 = gemm_launch(grad, mat2, s1, false, !t2);
+            g2 = gemm_launch(grad, mat1, s2, true, !t1);
+        }
         return {g1.view_as(saved[0]), g2.view_as(saved[1]), Tensor(), Tensor(), Tensor(), Tensor(), Tensor(),
                 Tensor(), Tensor(), Tensor()};
     }

@@ -269,6 +269,17 @@ int ba_gemm_softmax_static(int64_t nseg, int mode, int64_t *MList, int64_t *NLis
                            const void *B, void *out, int out_dtype, int64_t H, int64_t Dm1, int64_t Dm2, int64_t Dout,
                            float scale, ba_stream_t stream);
 
+/* Two calls of ba_varlen_gemm as ONE launch: (plan_a, transpose1 = 0, transpose2 = 1) and (plan_b, transpose1 = 1,
+ * transpose2 = 1), the layouts of the two products of the backward pass (dA = dS B over plan_a = the forward's
+ * metadata with N and K exchanged, dB = dS^T A over plan_b; reference: csrc/sparseBlockedAttention.cpp:52-72 makes the
+ * two calls one after the other).  Only where both would run as the 64 x 64 build of the kernel for transposed
+ * layouts with the summaries given (16-bit types, batches of short segments: there each product alone is a few rounds
+ * of short-lived workgroups); otherwise BA_ERR_UNSUPPORTED and nothing is launched: make the two calls instead. */
+int ba_varlen_gemm_two(int dtype, int64_t H, void *plan_a, const ba_plan_info *info_a, const void *A_a, const void *B_a,
+                       void *out_a, int64_t Dm1_a, int64_t Dm2_a, int64_t Dout_a, void *plan_b, const ba_plan_info *info_b,
+                       const void *A_b, const void *B_b, void *out_b, int64_t Dm1_b, int64_t Dm2_b, int64_t Dout_b,
+                       ba_stream_t stream);
+
 /* ba_plan_read on the buffer of ba_gemm_softmax_static (current device): the verdict of the LAST call of that entry
  * point on `stream` -- BA_ERR_BAD_METADATA with bad_segments / run_errors set when that call's metadata was
  * rejected or its totals did not match the sizes passed, in which case it wrote nothing.  Blocks like ba_plan_read

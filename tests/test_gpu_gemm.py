@@ -197,3 +197,36 @@ def test_unsupported_dtype_and_empty_calls(dev):
         capi.varlen_gemm(plan, x, x, x, 1, 32, 32, 16)
     e = torch.empty((0, 32), dtype=torch.float16, device=dev)
     capi.varlen_gemm(plan, e, e, torch.empty((0, 16), dtype=torch.float16, device=dev), 0, 32, 32, 16)
+
+
+def test_two_products_in_one_launch(dev):
+    # the backward pass's two products of a batch of short segments as ONE launch: the same bits as the two calls, and
+    # BA_ERR_UNSUPPORTED (nothing written) where the library wants two calls (tall segments: the 128 x 128 build)
+    rng = np.random.default_rng(61)
+    for nseg, top, dtype in ((90, 130, torch.float16), (33, 70, torch.bfloat16), (6, 900, torch.float16)):
+        M = rng.integers(1, top, nseg); N = rng.integers(1, top, nseg); K = rng.choice([8, 32, 64, 72, 128], nseg)
+        H = 3
+        A, B = random_operands(M, N, K, H, dtype, seed=nseg)
+        dS = torch.randn((H, int((M * N).sum()))).to(dtype)
+        Ad, Bd, dSd = A.to(dev), B.to(dev), dS.to(dev)
+        # dA = dS B: rows M, columns K, reduction N, B stored N x K = k-major; dB = dS^T A: rows N, columns K, reduction M
+        d_out, d_a, d_b = int((M * N).sum()), int((M * K).sum()), int((N * K).sum())
+        acc = lambda x: dev_i64(np.concatenate([[0], np.cumsum(x)]), dev)
+        plan_a = capi.plan_gemm(nseg, dev, dev_i64(M, dev), dev_i64(K, dev), dev_i64(N, dev), acc(M * N), acc(N * K), acc(M * K),
+                                mode=capi.META_GIVEN)
+        plan_b = capi.plan_gemm(nseg, dev, dev_i64(N, dev), dev_i64(K, dev), dev_i64(M, dev), acc(M * N), acc(M * K), acc(N * K),
+                                mode=capi.META_GIVEN)
+        plan_a.read(); plan_b.read()
+        one = [torch.full((H, d), float("nan"), dtype=dtype, device=dev) for d in (d_a, d_b)]
+        capi.varlen_gemm(plan_a, dSd, Bd, one[0], H, d_out, d_b, d_a, False, True)
+        capi.varlen_gemm(plan_b, dSd, Ad, one[1], H, d_out, d_a, d_b, True, True)
+        two = [torch.full((H, d), float("nan"), dtype=dtype, device=dev) for d in (d_a, d_b)]
+        ran = capi.varlen_gemm_two(plan_a, dSd, Bd, two[0], (d_out, d_b, d_a), plan_b, dSd, Ad, two[1], (d_out, d_a, d_b), H)
+        assert ran == (top < 200)
+        if ran:
+            assert torch.equal(one[0], two[0]) and torch.equal(one[1], two[1])
+            ref = oracle.varlen_gemm(dS.float().numpy(), B.float().numpy(), M, K, N, False, True, f64acc=True)
+            assert_scores_close(two[0], torch.from_numpy(ref), "dA")
+        else:
+            assert torch.isnan(two[0]).all() and torch.isnan(two[1]).all()
+
