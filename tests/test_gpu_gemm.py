@@ -229,4 +229,22 @@ def test_two_products_in_one_launch(dev):
             assert_scores_close(two[0], torch.from_numpy(ref), "dA")
         else:
             assert torch.isnan(two[0]).all() and torch.isnan(two[1]).all()
+    # sizes that do not match the second plan: that product writes nothing and its plan counts a run error, the
+    # first product is done all the same
+    M, N, K = (rng.integers(1, 60, 12) for _ in range(3))
+    K = 8 * (K // 8 + 1)
+    A, B = random_operands(M, N, K, H, torch.float16, seed=5)
+    dS = torch.randn((H, int((M * N).sum()))).half()
+    d_out, d_a, d_b = int((M * N).sum()), int((M * K).sum()), int((N * K).sum())
+    acc = lambda x: dev_i64(np.concatenate([[0], np.cumsum(x)]), dev)
+    plan_a = capi.plan_gemm(12, dev, dev_i64(M, dev), dev_i64(K, dev), dev_i64(N, dev), acc(M * N), acc(N * K), acc(M * K), mode=capi.META_GIVEN)
+    plan_b = capi.plan_gemm(12, dev, dev_i64(N, dev), dev_i64(K, dev), dev_i64(M, dev), acc(M * N), acc(M * K), acc(N * K), mode=capi.META_GIVEN)
+    plan_a.read(); plan_b.read()
+    out_a = torch.full((H, d_a), float("nan"), dtype=torch.float16, device=dev)
+    out_b = torch.full((H, d_b + 8), float("nan"), dtype=torch.float16, device=dev)
+    assert capi.varlen_gemm_two(plan_a, dS.to(dev), B.to(dev), out_a, (d_out, d_b, d_a), plan_b, dS.to(dev), A.to(dev), out_b,
+                                (d_out, d_a, d_b + 8), H)
+    torch.cuda.synchronize()
+    assert torch.isnan(out_b).all() and not torch.isnan(out_a).any()
+    assert plan_b.read(raise_on_bad=False).run_errors == 1 and plan_a.read().run_errors == 0
 
