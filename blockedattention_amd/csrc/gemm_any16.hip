@@ -409,8 +409,9 @@ __device__ __forceinline__ void any16_ring_round(__amdgpu_buffer_rsrc_t resX, __
 // bound by operand traffic out of L2 (a 64 x 64 step fetches 16 KiB for 32 matrix instructions), which the
 // 128 x 128 step halves per result.
 template <int DT, int RT, int CG, bool T1, bool T2>
-__device__ __forceinline__ void any16_stream_round(__amdgpu_buffer_rsrc_t resX, __amdgpu_buffer_rsrc_t resY, uint16_t *os, int M,
-                                                   int N, int K, int r0, unsigned char *any_lds) {
+__device__ __forceinline__ void any16_stream_rounds(__amdgpu_buffer_rsrc_t resX, __amdgpu_buffer_rsrc_t resY, uint16_t *os, int M,
+                                                    int N, int K, int first_round, int round_step, int rounds,
+                                                    unsigned char *any_lds) {
     constexpr int kRows = kAnyTile * RT, kCols = kAnyTile * CG;
     constexpr int kPitchXT = AnyBuf<kRows>::pitch_t, kPitchYT = AnyBuf<kCols>::pitch_t;
     constexpr int kBufBytes = AnyBuf<kRows>::bytes + AnyBuf<kCols>::bytes;
@@ -474,9 +475,15 @@ __device__ __forceinline__ void any16_stream_round(__amdgpu_buffer_rsrc_t resX, 
     // once instead of once per column block; only Y streams.
     const bool x_once = nkc <= 2;
     clear();
+    // The workgroup's rounds (first_round, first_round + round_step, ... below `rounds`) are ONE stream of steps: the
+    // loads of a round's first chunks are issued during the last steps of the round before, so only the first round
+    // of a workgroup waits for memory with nothing to do.
+    const int my_rounds = first_round < rounds ? (rounds - 1 - first_round) / round_step + 1 : 0;
+    const int total = my_rounds * steps;
     // a stage = the registers of one chunk in flight (plain vectors: the staging union only lives inside the calls)
     struct Stage { u32x4 x[RT][2], y[CG][2]; };
-    auto fetch = [&](Stage &st, int cb, int kc) __attribute__((always_inline)) {
+    auto fetch = [&](Stage &st, int round, int cb, int kc) __attribute__((always_inline)) {
+        const int r0 = round * kRows;
         if (!x_once || cb == 0) {
 #pragma unroll
             for (int i = 0; i < RT; ++i) {
@@ -490,15 +497,22 @@ __device__ __forceinline__ void any16_stream_round(__amdgpu_buffer_rsrc_t resX, 
             st.y[i][0] = l.v[0]; st.y[i][1] = l.v[1];
         }
     };
-    int f_cb = 0, f_kc = 0;                       // the chunk the next fetch takes
+    int f_round = first_round, f_cb = 0, f_kc = 0;        // the chunk the next fetch takes
     auto advance = [&]() {
-        if (++f_kc == nkc) { f_kc = 0; ++f_cb; }
+        if (++f_kc == nkc) {
+            f_kc = 0;
+            if (++f_cb == ncb) { f_cb = 0; f_round += round_step; }
+        }
     };
     Stage sa, sb;
-    if (steps > 0) { fetch(sa, f_cb, f_kc); advance(); }
-    if (steps > 1) { fetch(sb, f_cb, f_kc); advance(); }
-    int cb = 0, kc = 0;                           // the chunk being computed
-    auto do_step = [&](int step, Stage &st) __attribute__((always_inline)) {
+    if (total > 0) { fetch(sa, f_round, f_cb, f_kc); advance(); }
+    if (total > 1) { fetch(sb, f_round, f_cb, f_kc); advance(); }
+    int c_round = first_round, cb = 0, kc = 0;            // the chunk being computed
+    auto do_step = [&](int gs, Stage &st) __attribute__((always_inline)) {
+        const int step = cb * nkc + kc;                   // position inside the round: decides the buffers
+        const int r0 = c_round * kRows;
+        // a new round's X chunks go where the last one's lie: wait until every wavefront has read those
+        if (step == 0 && gs > 0) lds_barrier();
         unsigned char *buf = any_lds + (step & 1) * kBufBytes;
         unsigned char *xbuf = any_lds + (x_once ? kc : step & 1) * kBufBytes;
         if (!x_once || cb == 0) {
@@ -516,7 +530,7 @@ __device__ __forceinline__ void any16_stream_round(__amdgpu_buffer_rsrc_t resX, 
             put_chunk16<true, 4 * CG, kPitchYT>(l, t2, N, K, cb * kCols, kc * kAnyTile, buf + AnyBuf<kRows>::bytes,
                                                 tid + kAnyThreads * i);
         }
-        if (step + 2 < steps) { fetch(st, f_cb, f_kc); advance(); }   // in flight under two steps of matrix instructions
+        if (gs + 2 < total) { fetch(st, f_round, f_cb, f_kc); advance(); }   // in flight under two steps of matrix instructions
         // every wavefront has written its part of this chunk, and is done reading the chunk before last,
         // whose buffer the NEXT step's writes go to
         lds_barrier();
@@ -551,14 +565,18 @@ __device__ __forceinline__ void any16_stream_round(__amdgpu_buffer_rsrc_t resX, 
             for (int rt = 0; rt < RT; ++rt) acc[rt][t] = Elem<DT>::mfma(av[ks & 1][rt], bq[f % 3], acc[rt][t]);
         }
         if (kc == nkc - 1) store_block(cb, r0);
-        if (++kc == nkc) { kc = 0; ++cb; }
+        if (++kc == nkc) {
+            kc = 0;
+            if (++cb == ncb) { cb = 0; c_round += round_step; }
+        }
     };
-    for (int step = 0; step < steps; step += 2) {
-        do_step(step, sa);
-        if (step + 1 < steps) do_step(step + 1, sb);
+    for (int gs = 0; gs < total; gs += 2) {
+        do_step(gs, sa);
+        if (gs + 1 < total) do_step(gs + 1, sb);
     }
     if (nkc == 0)                                                  // K = 0: the result is zeros
-        for (int c = 0; c < ncb; ++c) store_block(c, r0);
+        for (int round = first_round; round < rounds; round += round_step)
+            for (int c = 0; c < ncb; ++c) store_block(c, round * kRows);
 }
 
 // RING: the kernel of the segments that any16_ring_segment accepts (128 x 128 build only); the other build of the pair
@@ -623,12 +641,13 @@ __device__ __forceinline__ void any16_workgroup(const RunArgs &a, unsigned block
     uint16_t *os = reinterpret_cast<uint16_t *>(a.out) + h * a.Dout + rec.offO;
     if (RING && threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->ring_groups, 1);
     const int rounds = (M + kRows - 1) / kRows;
-    for (int round = first_round; round < rounds; round += round_step) {
-        const int r0 = round * kRows;
-        if constexpr (RING) any16_ring_round<DT, T1, T2>(resX, resY, os, M, N, K, r0, any_lds);
-        else any16_stream_round<DT, RT, CG, T1, T2>(resX, resY, os, M, N, K, r0, any_lds);
-        // the next round's first chunks may take either buffer, and go where the rings are
-        if (round + round_step < rounds) lds_barrier();
+    if constexpr (RING) {
+        for (int round = first_round; round < rounds; round += round_step) {
+            any16_ring_round<DT, T1, T2>(resX, resY, os, M, N, K, round * kRows, any_lds);
+            if (round + round_step < rounds) lds_barrier();        // the next round's X chunks go where the rings are
+        }
+    } else {
+        any16_stream_rounds<DT, RT, CG, T1, T2>(resX, resY, os, M, N, K, first_round, round_step, rounds, any_lds);
     }
 }
 
@@ -685,6 +704,9 @@ int launch_gemm_any16(int dtype, const RunArgs &args, int64_t nseg, const ba_pla
     static const int tile_env = [] { const char *e = getenv("BLOCKEDATTN_ANY_TILE"); return e ? atoi(e) : 0; }();
     const bool big = tile_env ? tile_env == 128 : info && (int64_t)info->att_blocks64 >= 4 * (int64_t)info->nseg;
     const int64_t items = info ? (int64_t)(big ? info->att_blocks128 : info->att_blocks64) * args.H : 0;
+    // (one workgroup per existing round, not per (segment, head): a 64 x 64 x 64 step takes a workgroup about a
+    // microsecond whatever is in flight, so the rounds of a segment are worth more side by side than one after the
+    // other -- 512 segments of 16..256 rows: 20.8 us against 35 / 26 / 22 us with one / two / three workgroups per pair)
     if (info && items < (int64_t(1) << 31) - 1024) {
         if (items == 0) return BA_OK;                   // no segment has rows
         run.ride_slots = 1;

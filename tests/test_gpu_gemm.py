@@ -101,6 +101,12 @@ def test_transposed_layouts_of_tall_segments(dev, dtype, t1, t2):
     ring_rounds = sum(-(-m // 128) for m, n, k in zip(M, N, K) if k <= 128 and n >= 128)
     assert (plan.info.min_N, plan.info.min_K) == (100, 8)
     assert plan.read().ring_groups == 3 * H * ring_rounds
+    # without the host summary: the 64 x 64 build, four workgroups per (segment, head), each taking every fourth
+    # round as one stream of steps (the loads of a round's first chunks issued during the round before)
+    plan.info = None
+    out = torch.full((H, i.Dout), float("nan"), dtype=dtype, device=dev)
+    capi.varlen_gemm(plan, A.to(dev), B.to(dev), out, H, i.Dm1, i.Dm2, i.Dout, t1, t2)
+    assert_scores_close(out, ref, f"transpose {t1} {t2} without the summary")
 
 
 def test_ragged_edges_and_degenerate_segments(dev):
