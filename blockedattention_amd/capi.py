@@ -35,7 +35,7 @@ class PlanInfo(ctypes.Structure):
         ("bad_segments", ctypes.c_int32), ("run_errors", ctypes.c_int32), ("list_small", ctypes.c_int32), ("list_big", ctypes.c_int32), ("list_tile", ctypes.c_int32),
         ("list_rest", ctypes.c_int32), ("small_max_N", ctypes.c_int32), ("small_max_M", ctypes.c_int32),
         ("list_rows", ctypes.c_int32), ("att_blocks64", ctypes.c_int32), ("att_blocks128", ctypes.c_int32),
-        ("list_mini", ctypes.c_int32), ("list_pipe", ctypes.c_int32), ("pipe_groups", ctypes.c_int32), ("min_N", ctypes.c_int32), ("min_K", ctypes.c_int32), ("ring_groups", ctypes.c_int32),
+        ("list_mini", ctypes.c_int32), ("list_pipe", ctypes.c_int32), ("pipe_groups", ctypes.c_int32), ("min_N", ctypes.c_int32), ("min_K", ctypes.c_int32), ("ring_groups", ctypes.c_int32), ("wide_groups", ctypes.c_int32),
     ]
 
     def as_dict(self):

@@ -19,7 +19,9 @@ enum RunFlags : int {
     kFlagSmallToo = 128,   // strip kernel, 64 KiB launch: the slots from both_split on walk the main launch's list
     kFlagHeadFast = 256,   // strip kernel: grid (head, slot, z) instead of (slot, head, z)
     kFlagPipeToo = 512,    // tile kernel: the pipelined row-block kernel runs in the same call and takes its segments
-    kFlagRingToo = 1024    // any-layout GEMM: the ring kernel runs in the same call and takes its segments
+    kFlagRingToo = 1024,   // any-layout GEMM: the ring kernel runs in the same call and takes its segments
+    kFlagWideKToo = 2048,  // tile and row-block kernel: the row-block kernel's build for 128 < K <= 256 runs in the same call and takes its segments
+    kFlagRowsToo = 4096    // tile kernel: the row-block kernel runs in the same call and takes the large segments with K <= 128
 };
 
 struct RunArgs {
@@ -58,6 +60,9 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
 // BA_ERR_UNSUPPORTED when the plan summary is missing or does not fit; the caller then takes launch_tiles.
 int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
                      hipStream_t stream);
+// Its build for 128 < K <= 256 over the same list; workgroups of other segments leave at once.
+int launch_rowblocks_wide_k(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
+                            hipStream_t stream);
 // The pipelined row-block kernel (rowpipe_kernel.hip): the fused pair over the same list, two sweeps of adjacent
 // row blocks sharing one stream of B_g.  Same conditions as launch_rowblocks.
 int launch_rowpipe(int dtype, const RunArgs &args, int64_t slots, const ba_plan_info *info, hipStream_t stream);

@@ -108,7 +108,8 @@ struct PlanHeader {
     int32_t pipe_groups;     // bumped by every workgroup of the pipelined row-block kernel that found work in this plan
     int32_t min_N, min_K;    // smallest N and K over the segments that have rows and columns (0: there is none)
     int32_t ring_groups;     // bumped by every workgroup of the any-layout GEMM that wrote its rows through the LDS ring
-    int32_t pad_[13];
+    int32_t wide_groups;     // bumped by every workgroup of the row-block kernel's build for 128 < K <= 256 that found work
+    int32_t pad_[12];
 };
 static_assert(sizeof(PlanHeader) == 256, "PlanHeader must stay 256 bytes");
 
@@ -138,6 +139,11 @@ __host__ __device__ inline bool tile_segment(int kind, int N, int K) {
 // columns deep.
 __host__ __device__ inline bool pipe_segment(int kind, int N, int K) {
     return tile_segment(kind, N, K) && K <= 128 && N > 4 * 64;
+}
+// Segments of the tile list that the row-block kernel's build for 128 < K <= 256 takes (16-bit results) where the
+// call launches it.
+__host__ __device__ inline bool wide_k_segment(int kind, int N, int K) {
+    return tile_segment(kind, N, K) && K > 128 && K <= 256;
 }
 
 // Launch class (work list) of a segment of a GEMM plan, or -1 for none.

@@ -128,6 +128,7 @@ static int info_from_header(const PlanHeader &h, ba_plan_info *info) {
     info->pipe_groups = h.pipe_groups;
     info->min_N = h.min_N; info->min_K = h.min_K;
     info->ring_groups = h.ring_groups;
+    info->wide_groups = h.wide_groups;
     return (h.bad_segments || h.run_errors) ? BA_ERR_BAD_METADATA : BA_OK;
 }
 

@@ -83,9 +83,14 @@ __device__ __forceinline__ u32x4 ring_read16(const unsigned char *row, int pos) 
                  __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh)};
 }
 
-template <int DT, bool FUSED>
+// WIDE: the build for 128 < K <= 256.  A chunk of B_g then takes TWO stages (k below 128, k from 128 on), so the four
+// stages hold two chunks and a chunk is requested one iteration ahead instead of three; a wavefront keeps sixteen A
+// fragments per row tile.
+template <int DT, bool FUSED, bool WIDE>
 __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunArgs a, int zdim, int weave) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    constexpr int kSlots = WIDE ? kRbStages / 2 : kRbStages;      // chunks of B_g the stages hold
+    constexpr int kSlotStages = WIDE ? 2 : 1;
     const unsigned block = blockIdx.x;
     const int die = block % kDies, slot = block / kDies;
     // `weave` pairs of a die take turns in the die's slots (pair fastest, then the pair's workgroups)
@@ -131,8 +136,13 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
     if (!valid || !tile_segment(s.kind, s.N, s.K)) return;
     const int M = s.M, N = s.N, K = s.K;
     if (z0 * kRbRows >= M) return;
-    if (K > 128) {                                        // the launch was sized for another plan
-        if (z0 == 0 && threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
+    if constexpr (WIDE) {
+        if (K <= 128 || K > 256) return;                  // the other kernels of the call take it
+        if (threadIdx.x == 0) atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->wide_groups, 1);
+    } else if (K > 128) {
+        // the wide build or the tile kernel of the same call takes it; without them the launch was sized for another plan
+        if (!(a.flags & kFlagWideKToo) && z0 == 0 && threadIdx.x == 0)
+            atomicAdd(&reinterpret_cast<PlanHeader *>(a.plan)->run_errors, 1);
         return;
     }
     const int lane = lane_id(), j = lane & 15, rg = lane >> 4;
@@ -175,22 +185,29 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
         const int piece = (lane & 15) ^ (i & 15);
         fill_off[n] = (uint32_t)((4 * i + (lane >> 4)) * K + piece * 8) * 2u;
     }
-    const bool full_k = kpieces == 16;
-    auto fill = [&](int cbi, int stage) __attribute__((always_inline)) {
+    // `slot`: which of the kSlots chunk places of the stages; span sp of a chunk (k from 128 sp on) goes to stage
+    // kSlotStages slot + sp
+    auto fill = [&](int cbi, int slot) __attribute__((always_inline)) {
         const int cb = cbi * kRbCols;
-        // (wave-uniform by construction; pinned so that the assembly below always gets scalar registers)
-        const char *base = reinterpret_cast<const char *>((uintptr_t)uniform64((int64_t)(uintptr_t)(bseg + (size_t)cb * K * 2)));
-        const bool whole = full_k && cb + kRbCols <= N;      // every lane of every instruction has something to fetch
 #pragma unroll
-        for (int n = 0; n < kRbFillInsts; ++n) {
-            const uint32_t dst = (uint32_t)uniform((int)(uint32_t)(uintptr_t)(lds + stage * kRbStageBytes + (wave + kRbWaves * n) * 1024));
-            if (whole) {
-                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                             :: "v"(fill_off[n]), "s"(base), "s"(dst) : "memory", "m0");
-            } else if (cb + 4 * (wave + kRbWaves * n) + (lane >> 4) < N &&
-                       ((lane & 15) ^ ((wave + kRbWaves * n) & 15)) < kpieces) {
-                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                             :: "v"(fill_off[n]), "s"(base), "s"(dst) : "memory", "m0");
+        for (int sp = 0; sp < kSlotStages; ++sp) {
+            // (wave-uniform by construction; pinned so that the assembly below always gets scalar registers)
+            const char *base = reinterpret_cast<const char *>(
+                (uintptr_t)uniform64((int64_t)(uintptr_t)(bseg + (size_t)cb * K * 2 + 256 * sp)));
+            const int span_pieces = kpieces - 16 * sp;          // pieces of a row that this span holds (at most 16 of them)
+            const bool whole = span_pieces >= 16 && cb + kRbCols <= N;      // every lane of every instruction has something to fetch
+#pragma unroll
+            for (int n = 0; n < kRbFillInsts; ++n) {
+                const uint32_t dst = (uint32_t)uniform(
+                    (int)(uint32_t)(uintptr_t)(lds + (slot * kSlotStages + sp) * kRbStageBytes + (wave + kRbWaves * n) * 1024));
+                if (whole) {
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                                 :: "v"(fill_off[n]), "s"(base), "s"(dst) : "memory", "m0");
+                } else if (cb + 4 * (wave + kRbWaves * n) + (lane >> 4) < N &&
+                           ((lane & 15) ^ ((wave + kRbWaves * n) & 15)) < span_pieces) {
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                                 :: "v"(fill_off[n]), "s"(base), "s"(dst) : "memory", "m0");
+                }
             }
         }
     };
@@ -199,7 +216,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) boff[ks] = 1024 * j + 16 * ((4 * ks + rg) ^ j);
 
-    // KS = k-steps of 32 the matrix instructions run over: 2 for K <= 64, else 4 (fragments past K are zeros)
+    // KS = k-steps of 32 the matrix instructions run over: 2 for K <= 64, 4 for K <= 128, 8 in the WIDE build (fragments past K are zeros)
     auto run = [&](auto ks_c) __attribute__((always_inline)) {
     constexpr int KS = decltype(ks_c)::value;
     for (int rb = z0; rb * kRbRows < M; rb += zdim) {
@@ -244,7 +261,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
             }
             if (threadIdx.x == 0) { flags[0] = 0; flags[1] = 0; }
             int f_cbi = 0;                               // chunk (inside its sweep) of the next fill
-            for (int k = 0; k < kRbStages - 1; ++k)
+            for (int k = 0; k < kSlots - 1; ++k)
                 if (k < total) {
                     fill(f_cbi, k);
                     if (++f_cbi == ncb) f_cbi = 0;
@@ -334,8 +351,8 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                 constexpr int MODE = decltype(mode_c)::value;
                 constexpr bool WT = decltype(wt_c)::value;       // sweep 1 only: the chunk has columns that do not exist
                 constexpr int b = decltype(buf_c)::value, pb = 1 - b;
-                constexpr int EPM = 32 / (8 * KS);            // score elements per matrix instruction
-                const unsigned char *sb = lds + stage * kRbStageBytes;
+                constexpr int EPM = KS == 2 ? 2 : 1;          // score elements per matrix instruction (KS = 8: of the first four k-steps)
+                const unsigned char *sb = lds + stage * (kSlotStages * kRbStageBytes);      // (stage: the chunk's slot)
                 const int cbp = cbi_prev * kRbCols;
                 float w[4];                                   // 0 for columns that do not exist (ragged last chunk)
 #pragma unroll
@@ -376,7 +393,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                     if (ks + 1 < KS) {
 #pragma unroll
                         for (int ct = 0; ct < 4; ++ct)
-                            bf[(ks + 1) & 1][ct] = *reinterpret_cast<const u32x4 *>(sb + boff[ks + 1] + 256 * ct);
+                            bf[(ks + 1) & 1][ct] = *reinterpret_cast<const u32x4 *>(sb + ((ks + 1) >> 2) * kRbStageBytes + boff[(ks + 1) & 3] + 256 * ct);
                     }
                     auto group = [&](auto qd_c) {
                         constexpr int qd = decltype(qd_c)::value, rt = qd >> 2, ct = qd & 3;
@@ -385,7 +402,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                         if constexpr (MODE != 0) {
                             if (ks == 0) { if constexpr (EPM == 1) element(std::integral_constant<int, 0 * 8 + qd>{}); else { element(std::integral_constant<int, (0 * 8 + qd) * 2>{}); element(std::integral_constant<int, (0 * 8 + qd) * 2 + 1>{}); } }
                             if (ks == 1) { if constexpr (EPM == 1) element(std::integral_constant<int, 1 * 8 + qd>{}); else { element(std::integral_constant<int, (1 * 8 + qd) * 2>{}); element(std::integral_constant<int, (1 * 8 + qd) * 2 + 1>{}); } }
-                            if constexpr (KS == 4) {
+                            if constexpr (KS >= 4) {
                                 if (ks == 2) element(std::integral_constant<int, 2 * 8 + qd>{});
                                 if (ks == 3) element(std::integral_constant<int, 3 * 8 + qd>{});
                             }
@@ -463,14 +480,14 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
             using I2 = std::integral_constant<int, 2>;
             auto iterate = [&](auto par_c, auto mode_c, auto wt_c, auto later_c, auto sync_c, int it, int cbi_prev) __attribute__((always_inline)) {
                 if constexpr (decltype(sync_c)::value) {
-                    if constexpr (kRbStages == 2) {
+                    if constexpr (kSlots == 2) {
                         wait_vm<decltype(later_c)::value>();
                     } else {
                         // fill of chunk `it`: requested kRbStages - 1 iterations ago; the fills requested since and the
                         // window stores of those iterations (each behind its iteration's fill) may stay in flight
                         int later = 0;
 #pragma unroll
-                        for (int k = 1; k <= kRbStages - 2; ++k) {
+                        for (int k = 1; k <= kSlots - 2; ++k) {
                             // (the fill of a ragged last chunk is not counted: its instructions for rows past N
                             // are skipped altogether, so fewer than kRbFillInsts may have been issued)
                             const int c = it + k, last = c == ncb - 1 || c == 2 * ncb - 1;
@@ -479,7 +496,7 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                         if (active) {
                             const int first_store = (FUSED ? ncb : 0) + 1;    // first iteration whose body stores (interior chunks: 4 instructions)
 #pragma unroll
-                            for (int back = 1; back <= kRbStages - 1; ++back) {
+                            for (int back = 1; back <= kSlots - 1; ++back) {
                                 const int cb2 = it - back - first_store;      // chunk that iteration stored
                                 if (cb2 >= 1 && cb2 < ncb - 1) later += kRbStoreInsts;
                             }
@@ -488,13 +505,13 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
                     }
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                    if (it + kRbStages - 1 < total) {
-                        fill(f_cbi, (it + kRbStages - 1) & (kRbStages - 1));
+                    if (it + kSlots - 1 < total) {
+                        fill(f_cbi, (it + kSlots - 1) & (kSlots - 1));
                         if (++f_cbi == ncb) f_cbi = 0;
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (active) chunk_body(mode_c, wt_c, par_c, it & (kRbStages - 1), cbi_prev);   // it % 2 == par
+                if (active) chunk_body(mode_c, wt_c, par_c, it & (kSlots - 1), cbi_prev);   // it % 2 == par
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             };
             const bool ragged = (N & (kRbCols - 1)) != 0;
@@ -543,24 +560,27 @@ __global__ __launch_bounds__(kRbThreads, 8 / kRbWaves) void rowblock_kernel(RunA
         }
     }
     };
-    if (K <= 64) run(std::integral_constant<int, 2>{});
+    if constexpr (WIDE) run(std::integral_constant<int, 8>{});
+    else if (K <= 64) run(std::integral_constant<int, 2>{});
     else run(std::integral_constant<int, 4>{});
 }
 
-template <int DT, bool FUSED>
+template <int DT, bool FUSED, bool WIDE = false>
 static int launch_rb(const RunArgs &args, unsigned groups, int zdim, int weave, hipStream_t stream) {
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&rowblock_kernel<DT, FUSED>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&rowblock_kernel<DT, FUSED, WIDE>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes);
     if (attr != hipSuccess) return BA_ERR_LAUNCH;
-    hipLaunchKernelGGL((rowblock_kernel<DT, FUSED>), dim3(groups), dim3(kRbThreads), kRbLdsBytes, stream, args, zdim, weave);
+    hipLaunchKernelGGL((rowblock_kernel<DT, FUSED, WIDE>), dim3(groups), dim3(kRbThreads), kRbLdsBytes, stream, args, zdim, weave);
     return BA_OK;
 }
 
 // Launches the row-block kernel over (list entry, head, row block of 256 rows).  Needs the plan summary:
-// every segment must have K <= 128 (the A fragments of a wavefront's rows stay in registers).
-int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
-                     hipStream_t stream) {
-    if (!info || info->max_K > 128 || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
+// every segment must have K <= 128 (the A fragments of a wavefront's rows stay in registers); wide: the build for
+// 128 < K <= 256, which passes over the segments outside that range.
+static int launch_rowblocks_any(bool wide, int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
+                                hipStream_t stream) {
+    if (!info || (args.flags & kFlagOutF32)) return BA_ERR_UNSUPPORTED;
+    if (wide ? info->max_K <= 128 : (info->max_K > 128 && !(args.flags & kFlagWideKToo))) return BA_ERR_UNSUPPORTED;
     if (slots <= 0) return BA_OK;
     int64_t pairs = (slots * args.H + kDies - 1) / kDies * kDies;   // (entry, head) pairs, padded to whole dies
     // Workgroups per pair Z (workgroup z of a pair takes its row blocks z, z + Z, ..) and pairs of a die that take
@@ -583,13 +603,31 @@ int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, c
     const int64_t groups = pairs * z;
     if (pairs > (int64_t(1) << 30) || groups > (int64_t(1) << 31) - 1) return BA_ERR_UNSUPPORTED;
     int st;
-    if (dtype == BA_F16) st = fused ? launch_rb<0, true>(args, (unsigned)groups, (int)z, (int)weave, stream)
-                                    : launch_rb<0, false>(args, (unsigned)groups, (int)z, (int)weave, stream);
-    else if (dtype == BA_BF16) st = fused ? launch_rb<1, true>(args, (unsigned)groups, (int)z, (int)weave, stream)
-                                          : launch_rb<1, false>(args, (unsigned)groups, (int)z, (int)weave, stream);
-    else return BA_ERR_UNSUPPORTED;
+    const unsigned g = (unsigned)groups;
+    const int zi = (int)z, wi = (int)weave;
+    if (dtype == BA_F16) {
+        if (wide) st = fused ? launch_rb<0, true, true>(args, g, zi, wi, stream) : launch_rb<0, false, true>(args, g, zi, wi, stream);
+        else st = fused ? launch_rb<0, true>(args, g, zi, wi, stream) : launch_rb<0, false>(args, g, zi, wi, stream);
+    } else if (dtype == BA_BF16) {
+        if (wide) st = fused ? launch_rb<1, true, true>(args, g, zi, wi, stream) : launch_rb<1, false, true>(args, g, zi, wi, stream);
+        else st = fused ? launch_rb<1, true>(args, g, zi, wi, stream) : launch_rb<1, false>(args, g, zi, wi, stream);
+    } else {
+        return BA_ERR_UNSUPPORTED;
+    }
     if (st != BA_OK) return st;
     return hipGetLastError() == hipSuccess ? BA_OK : BA_ERR_LAUNCH;
+}
+
+int launch_rowblocks(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
+                     hipStream_t stream) {
+    return launch_rowblocks_any(false, dtype, fused, args, slots, info, stream);
+}
+
+// The build for 128 < K <= 256 over the same list: the workgroups of every other segment leave at once (the caller
+// launches the kernels that take those, with kFlagWideKToo).
+int launch_rowblocks_wide_k(int dtype, int fused, const RunArgs &args, int64_t slots, const ba_plan_info *info,
+                            hipStream_t stream) {
+    return launch_rowblocks_any(true, dtype, fused, args, slots, info, stream);
 }
 
 }  // namespace ba

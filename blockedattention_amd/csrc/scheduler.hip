@@ -363,6 +363,7 @@ __global__ __launch_bounds__(kSchedThreads) void schedule_kernel(SchedArgs a) {
         h->min_N = rInvN ? INT32_MAX - rInvN : 0;
         h->min_K = rInvK ? INT32_MAX - rInvK : 0;
         h->ring_groups = 0;
+        h->wide_groups = 0;
         plan_rowblocks(a.plan, nseg, 0)[nseg] = base32[kPfxAtt64];     // zero for softmax plans
         plan_rowblocks(a.plan, nseg, 1)[nseg] = base32[kPfxAtt128];
         if (a.mailbox) {

@@ -386,6 +386,8 @@ __device__ __forceinline__ void tile_block(const RunArgs &a, int zdim, unsigned 
     const int kind = s.kind;
     if (!tile_segment(kind, s.N, s.K)) return;
     if ((a.flags & kFlagPipeToo) && pipe_segment(kind, s.N, s.K)) return;      // the other kernel of this call takes it
+    if ((a.flags & kFlagWideKToo) && wide_k_segment(kind, s.N, s.K)) return;   // likewise
+    if ((a.flags & kFlagRowsToo) && s.K <= 128) return;
     tile_rows<DT, FUSED, F32OUT>(a, s, z0, zdim, lds);
 }
 

@@ -24,9 +24,15 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
     if (slots <= 0) return BA_OK;
     RunArgs targs = args;
     static const int use_pipe = [] { const char *e = getenv("BLOCKEDATTN_ROWPIPE"); return e ? atoi(e) : 1; }();
-    if (use_rowblocks && fused && !use_pipe && info && info->max_K <= 128 && !(args.flags & kFlagOutF32))
+    static const int use_wide_k = [] { const char *e = getenv("BLOCKEDATTN_ROWBLOCK_WIDE_K"); return e ? atoi(e) : 1; }();
+    const bool rows_ok = use_rowblocks && !(args.flags & kFlagOutF32);      // 16-bit results: the row-block kernels
+    // Large segments with 128 < K <= 256: the row-block kernel's build for them, where the summary says the batch may
+    // hold some; the kernels launched beside it pass over them.
+    const bool wide_ok = rows_ok && use_wide_k && info && info->max_K > 128;
+    bool all_taken = false;                                // nothing left for the tile kernel
+    if (rows_ok && fused && !use_pipe && info && info->max_K <= 128)
         return launch_rowblocks(dtype, fused, args, slots, info, stream);     // the kernel before the pipelined one
-    if (use_rowblocks && fused && use_pipe && !(args.flags & kFlagOutF32)) {
+    if (rows_ok && fused && use_pipe) {
         // The fused pair with 16-bit results: every segment with K <= 128 goes to the pipelined row-block kernel,
         // the others stay here.  The plan counts the former (list_pipe); without the summary both kernels are
         // launched over the whole list and each workgroup keeps to its own kind of segment.
@@ -40,8 +46,29 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
                 return st;
             }
         }
-    } else if (use_rowblocks && !fused && info && info->max_K <= 128) {
-        return launch_rowblocks(dtype, fused, args, slots, info, stream);
+    } else if (rows_ok && !fused && info) {
+        // The product alone: the row-block kernel for K <= 128, its wide build for K <= 256, the tile kernel beyond.
+        if (info->max_K <= 128) return launch_rowblocks(dtype, fused, args, slots, info, stream);
+        if (wide_ok) {
+            all_taken = info->max_K <= 256;
+            if (info->min_K <= 128) {
+                RunArgs na = args;
+                na.flags |= kFlagWideKToo;
+                const int st = launch_rowblocks(dtype, fused, na, slots, info, stream);
+                if (st == BA_OK) targs.flags |= kFlagRowsToo | kFlagQuiet;
+                else if (st != BA_ERR_UNSUPPORTED) return st;
+                else all_taken = false;
+            }
+        }
+    }
+    if (wide_ok) {
+        const int st = launch_rowblocks_wide_k(dtype, fused, targs, slots, info, stream);
+        if (st == BA_OK) {
+            if (all_taken) return BA_OK;
+            targs.flags |= kFlagWideKToo | kFlagQuiet;
+        } else if (st != BA_ERR_UNSUPPORTED) {
+            return st;
+        }
     }
     int64_t z = 4;
     if (info)

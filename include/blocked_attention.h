@@ -95,6 +95,9 @@ typedef struct ba_plan_info {
      * N >= 128) since the plan was built */
     int32_t min_N, min_K;
     int32_t ring_groups;
+    /* workgroups of the row-block kernel's build for 128 < K <= 256 (large segments, 16-bit results, whole-line
+     * stores) that have found work in this plan since it was built */
+    int32_t wide_groups;
 } ba_plan_info;
 
 const char *ba_status_string(int status);

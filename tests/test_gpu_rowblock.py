@@ -1,7 +1,8 @@
-"""Large segments with K <= 128 (the row-block kernels: 256 rows per workgroup or per wavefront set, 64 columns at
-a time, results through an LDS ring into line-aligned stores; the fused pair runs the two sweeps of adjacent row
-blocks side by side on one stream of B_g) against the oracle: every line phase, ragged rows and columns, every
-reduction length, the overflow path of the first sweep, GEMM alone and fused."""
+"""Large segments with K <= 256 (the row-block kernels: 256 rows per workgroup or per wavefront set, 64 columns at
+a time, results through an LDS ring into line-aligned stores; the fused pair with K <= 128 runs the two sweeps of
+adjacent row blocks side by side on one stream of B_g; 128 < K <= 256 takes a build with two LDS stages per chunk)
+against the oracle: every line phase, ragged rows and columns, every reduction length, the overflow path of the
+first sweep, GEMM alone and fused."""
 import numpy as np
 import pytest
 import torch
@@ -129,8 +130,9 @@ def test_nearly_empty_last_row_block_under_load(dev):
 
 
 def test_k_zero_in_the_tile_kernel(dev):
-    # without the host summary, and next to a K = 136 segment, the large segments run in the tile kernel: K = 0
-    # has no operand bytes there either, and the rows are zeros (product) or 1/N (fused pair)
+    # without the host summary the large segments run in the tile kernel, and so do large segments of 256 columns
+    # or fewer in a fused call: K = 0 has no operand bytes there either, and the rows are zeros (product) or 1/N
+    # (fused pair); the K = 136 neighbour takes the row-block kernel's wide build
     run_all(dev, [40, 200, 70], [300, 130, 260], [0, 0, 64], 2, torch.float16, 0.2, summary=False)
     run_all(dev, [40, 200, 70], [300, 130, 260], [0, 0, 136], 2, torch.bfloat16, 0.2)
 
@@ -149,13 +151,14 @@ def fused_only(dev, M, N, K, H, dtype, scale, summary, seed=0, out_dtype=None):
 
 
 def test_the_pipelined_kernel_is_chosen_segment_by_segment(dev):
-    # K = 136, 160 and 256 keep a segment in the tile kernel; its neighbours with K <= 128 still take the pipelined
-    # row-block kernel, in the same call (the plan counts them, the kernel counts the workgroups that worked)
+    # K = 136, 160 and 256 send a segment to the row-block kernel's wide build; its neighbours with K <= 128 still take
+    # the pipelined row-block kernel, in the same call (the plan counts them, the kernels count the workgroups that worked)
     M = [300, 520, 100, 260, 700, 64]; N = [400, 300, 1000, 263, 513, 200]; K = [128, 136, 64, 160, 8, 256]
     for dtype in (torch.float16, torch.bfloat16):
         info = fused_only(dev, M, N, K, 2, dtype, 0.13, summary=True, seed=3)
         assert info.list_tile == 6 and info.list_pipe == 3
         assert info.pipe_groups >= 3 * 2                      # at least one workgroup per eligible segment and head
+        assert info.wide_groups >= 3 * 2
 
 
 def test_the_pipelined_kernel_runs_without_the_host_summary(dev):
@@ -173,3 +176,64 @@ def test_fp32_probabilities_of_large_segments_stay_in_the_tile_kernel(dev):
     info = fused_only(dev, [300, 260], [400, 263], [128, 96], 2, torch.bfloat16, 0.2, summary=True, seed=7,
                       out_dtype=torch.float32)
     assert info.list_pipe == 2 and info.pipe_groups == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reduction_lengths_between_128_and_256(dev, dtype):
+    # every multiple of 8 that needs the second span, widths at every phase, heights around 256 and 32 rows;
+    # neighbours with K <= 128 and K > 256 go to the other kernels of the same call
+    M = [300, 256, 257, 1, 40, 33, 513, 31, 100, 90]; N = [257, 300, 1000, 3000, 320, 321, 263, 384, 300, 290]
+    K = [136, 256, 160, 200, 248, 144, 192, 232, 128, 264]
+    plan = run_all(dev, M, N, K, 3, dtype, 0.11, seed=7, sigma=0.5)
+    info = plan.read()
+    assert info.list_tile == len(M)
+    # GEMM and fused call: at least one workgroup per eligible segment and head in each
+    assert info.wide_groups >= 2 * 8 * 3
+
+
+def test_widths_modulo_the_chunk_and_negative_scale(dev):
+    N = np.concatenate([np.arange(257, 321, 3), [448, 449, 511, 512, 513]]); M = np.full(N.size, 37); K = np.full(N.size, 136)
+    K[::2] = 256
+    run_all(dev, M, N, K, 1, torch.float16, 0.3, seed=3, check_softmax=False, sigma=0.5)
+    run_all(dev, M[::3], N[::3], K[::3], 2, torch.bfloat16, -0.2, seed=4, check_softmax=False, sigma=0.5)
+
+
+def test_overflow_of_the_first_sweep(dev):
+    M = np.array([100, 64]); N = np.array([700, 300]); K = np.array([256, 160])
+    A, B = random_operands(M, N, K, 2, torch.float16, seed=11)
+    A = A.abs() * 0.7 + 0.7; B = B.abs()
+    Bs = B[:, :700 * 256].reshape(2, 700, 256)
+    Bs[:, :64] *= 0.01
+    Bs[:, 300:310] *= 4
+    plan = make_plan(dev, M, N, K)
+    i = plan.info
+    out = torch.full((2, i.Dout), float("nan"), dtype=torch.float16, device=dev)
+    capi.gemm_softmax(plan, A.to(dev), B.to(dev), out, 2, i.Dm1, i.Dm2, i.Dout, 1.0)
+    assert_probs_close(out, oracle.per_segment_torch(A, B, M, N, K, 1.0), "overflow path")
+    info = plan.read()
+    assert info.run_errors == 0 and info.wide_groups >= 4
+
+
+def test_many_heads_and_tall_segments(dev):
+    M = np.array([1267, 523, 11, 290]); N = np.array([1483, 2571, 900, 2594]); K = np.array([256, 136, 64, 200])
+    for rep in range(2):
+        plan = run_all(dev, M, N, K, 8, torch.bfloat16, 0.05, seed=21 + rep, sigma=0.5, check_softmax=False)
+    assert plan.read().wide_groups > 0
+
+
+def test_the_product_alone_is_routed_segment_by_segment(dev):
+    # K <= 128 to the row-block kernel, 128 < K <= 256 to its wide build, K > 256 to the tile kernel, in one call
+    M = [300, 520, 100, 260, 700, 64]; N = [400, 300, 1000, 263, 513, 200]; K = [128, 136, 64, 160, 8, 264]
+    plan = run_all(dev, M, N, K, 2, torch.bfloat16, 0.13, seed=3, sigma=0.5, check_softmax=False)
+    assert plan.read().wide_groups >= 2 * 2 * 2
+    # nothing beyond K = 256: the tile kernel is not launched for the product
+    plan = run_all(dev, M[:5], N[:5], K[:5], 2, torch.float16, 0.13, seed=4, sigma=0.5, check_softmax=False)
+    assert plan.read().wide_groups >= 2 * 2 * 2
+    # only wide segments
+    plan = run_all(dev, [300, 64], [400, 300], [256, 136], 2, torch.float16, 0.2, seed=5, sigma=0.5)
+    assert plan.read().wide_groups >= 2 * 2 * 2
+
+
+def test_without_the_summary_the_tile_kernel_takes_them(dev):
+    plan = run_all(dev, [300, 100], [400, 300], [256, 136], 2, torch.float16, 0.2, summary=False, sigma=0.5)
+    assert plan.read().wide_groups == 0
