@@ -29,7 +29,8 @@ int launch_tiles(int dtype, int fused, const RunArgs &args, int64_t slots, const
     // Large segments with 128 < K <= 256: the row-block kernel's build for them, where the summary says the batch may
     // hold some; the kernels launched beside it pass over them.
     const bool wide_ok = rows_ok && use_wide_k && info && info->max_K > 128;
-    bool all_taken = false;                                // nothing left for the tile kernel
+    // nothing left for the tile kernel: every large segment has 128 < K <= 256 (the product alone: see below)
+    bool all_taken = wide_ok && info->min_K > 128 && info->max_K <= 256;
     if (rows_ok && fused && !use_pipe && info && info->max_K <= 128)
         return launch_rowblocks(dtype, fused, args, slots, info, stream);     // the kernel before the pipelined one
     if (rows_ok && fused && use_pipe) {

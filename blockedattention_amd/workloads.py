@@ -64,8 +64,8 @@ class Workload:
         return a.to(dtype), b.to(dtype)
 
 
-def make(cfg, seed=0):
-    """cfg in 1..5 -> Workload."""
+def make(cfg, seed=0, k=None):
+    """cfg in 1..5 -> Workload.  k: configuration 5 with another reduction length (the name says which)."""
     rng = np.random.default_rng(seed)
     i64 = np.int64
     if cfg == 1:
@@ -87,6 +87,7 @@ def make(cfg, seed=0):
         return Workload("cfg4_nonsquare_512seg_mn16-256_k32-128", M, N, K, 1, torch.float16, 1.0, "uniform")
     if cfg == 5:
         n = rng.integers(1024, 4097, 16).astype(i64)
-        return Workload("cfg5_large_16seg_x16h_n1024-4096_k128", n, n.copy(), np.full(16, 128, i64), 16,
-                        torch.bfloat16, 128 ** -0.5, "normal", sigma=128 ** -0.5)
+        k = 128 if k is None else int(k)
+        return Workload(f"cfg5_large_16seg_x16h_n1024-4096_k{k}", n, n.copy(), np.full(16, k, i64), 16,
+                        torch.bfloat16, k ** -0.5, "normal", sigma=k ** -0.5)
     raise ValueError("cfg must be 1..5")
