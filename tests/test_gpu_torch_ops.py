@@ -151,8 +151,17 @@ def test_repeated_metadata_reuses_the_schedule(dev):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_autograd_16bit_through_the_any_layout_gemms(dev, dtype):
     # dA = dS B (reduction over N) and dB = dS^T A (over M) with N, M that are not multiples of 8
+    autograd_16bit(dev, dtype, [5, 33, 16, 130], [7, 20, 64, 257], [8, 16, 24, 64])
+
+
+def test_autograd_16bit_large_segments_of_every_reduction_length(dev):
+    # forward: the row-block kernel (K <= 128), its wide build (K <= 256) and the tile kernel (beyond) in one call;
+    # backward: products with 300..400 columns and reductions over them
+    autograd_16bit(dev, torch.bfloat16, [300, 130, 40, 280], [400, 300, 257, 310], [256, 136, 64, 264])
+
+
+def autograd_16bit(dev, dtype, M, N, K):
     import blockedAttention
-    M, N, K = [5, 33, 16, 130], [7, 20, 64, 257], [8, 16, 24, 64]
     g = torch.Generator().manual_seed(4)
     A0 = torch.randn((2, int(np.dot(M, K))), generator=g).to(dtype); B0 = torch.randn((2, int(np.dot(N, K))), generator=g).to(dtype)
     ML, NL, KL = dl(M, dev), dl(N, dev), dl(K, dev)
